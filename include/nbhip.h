@@ -1,0 +1,169 @@
+/*
+ * nbhip.h - C ABI of libnbhip.so: the MI355X (gfx950) back end of the numba-cuda
+ * data-parallel array library (reduce / transpose / xoroshiro128+ and the device
+ * memory, stream and event plumbing underneath them).
+ *
+ * The reference has no C boundary for this path: its Python layer reaches the
+ * CUDA driver through cuda.bindings and JIT-compiles its kernels.  Each entry
+ * point below names the reference interface it stands in for; paths are relative
+ * to numba_cuda/numba/cuda/ in NVIDIA/numba-cuda 0.30.4.
+ *
+ * Conventions
+ *   - every function returns a hipError_t as int; 0 is success; nothing throws
+ *   - all pointers are plain host or device addresses, sizes are in bytes unless
+ *     stated otherwise, strides are in bytes and may be negative
+ *   - nbh_stream_t is a hipStream_t; NULL is the legacy default stream
+ *   - the library never frees or reallocates caller memory; lifetimes of buffers
+ *     passed to asynchronous calls are the caller's to keep
+ *   - functions are re-entrant; the current device is per host thread
+ */
+#ifndef NBHIP_H
+#define NBHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *nbh_stream_t;
+typedef void *nbh_event_t;
+
+#define NBH_VERSION 1
+
+/* element types understood by nbh_reduce */
+enum nbh_dtype {
+    NBH_I8 = 0, NBH_I16 = 1, NBH_I32 = 2, NBH_I64 = 3,
+    NBH_U8 = 4, NBH_U16 = 5, NBH_U32 = 6, NBH_U64 = 7,
+    NBH_F32 = 8, NBH_F64 = 9,
+    NBH_DTYPE_COUNT = 10
+};
+
+/* binary operators understood by nbh_reduce.  Semantics are those the reference's
+ * JIT gives the Python functor (cpython/builtins.py:224-269):
+ *   ADD a + b, MUL a * b      native arithmetic, integers wrap modulo 2^bits
+ *   MAX b if b > a else a,  MIN b if b < a else a */
+enum nbh_op { NBH_ADD = 0, NBH_MUL = 1, NBH_MAX = 2, NBH_MIN = 3, NBH_OP_COUNT = 4 };
+
+/* ---- library / device ---------------------------------------------------- */
+
+int nbh_version(void);
+
+/* cudadrv/driver.py:245-419 Driver (error checking): name / text of an error code */
+const char *nbh_error_name(int code);
+const char *nbh_error_string(int code);
+
+/* cudadrv/driver.py:385-388 get_device_count */
+int nbh_device_count(int *count);
+/* cudadrv/devices.py:101-187 _Runtime (per-thread current context) */
+int nbh_set_device(int dev);
+int nbh_get_device(int *dev);
+/* cudadrv/driver.py:470-587 Device: name, attributes looked up by the CUDA
+ * attribute name without its CU_DEVICE_ATTRIBUTE_ prefix (:509-517), e.g.
+ * "MAX_THREADS_PER_BLOCK", "MULTIPROCESSOR_COUNT", "WARP_SIZE".  Unknown names
+ * return hipErrorInvalidValue. */
+int nbh_device_name(int dev, char *buf, int buflen);
+int nbh_device_attr(int dev, const char *name, int *value);
+/* cudadrv/driver.py:1095-1097 Context.get_memory_info */
+int nbh_mem_info(size_t *free_bytes, size_t *total_bytes);
+/* cudadrv/driver.py:1282-1283 Context.synchronize */
+int nbh_device_synchronize(void);
+
+/* ---- memory --------------------------------------------------------------- */
+
+/* cudadrv/driver.py:891-902 NumbaCUDAMemoryManager.memalloc (cuMemAlloc) and the
+ * cuMemFree its finalizer queues (:1316-1325) */
+int nbh_malloc(void **dptr, size_t nbytes);
+int nbh_free(void *dptr);
+/* cudadrv/driver.py:747-779 memhostalloc (cuMemHostAlloc / cuMemFreeHost).
+ * flags: bit 0 portable, bit 1 device-mapped, bit 2 write-combined */
+int nbh_host_alloc(void **hptr, size_t nbytes, unsigned flags);
+int nbh_host_free(void *hptr);
+/* cudadrv/driver.py:781-817 mempin (cuMemHostRegister / cuMemHostUnregister) */
+int nbh_host_register(void *hptr, size_t nbytes, unsigned flags);
+int nbh_host_unregister(void *hptr);
+/* cudadrv/driver.py:1735-1770 MappedMemory (cuMemHostGetDevicePointer) */
+int nbh_host_get_device_pointer(void **dptr, void *hptr);
+/* cudadrv/driver.py:2496-2506 device_extents (cuMemGetAddressRange) */
+int nbh_mem_address_range(void **base, size_t *size, void *dptr);
+
+/* cudadrv/driver.py:2625-2670 host_to_device / device_to_host / device_to_device:
+ * stream == NULL selects the synchronous copy, any other stream the asynchronous
+ * one, exactly as the reference picks cuMemcpyXtoY vs cuMemcpyXtoYAsync */
+int nbh_memcpy_h2d(void *dst, const void *src, size_t nbytes, nbh_stream_t stream);
+int nbh_memcpy_d2h(void *dst, const void *src, size_t nbytes, nbh_stream_t stream);
+int nbh_memcpy_d2d(void *dst, const void *src, size_t nbytes, nbh_stream_t stream);
+/* cudadrv/driver.py:2673-2704 device_memset (cuMemsetD8 / cuMemsetD8Async) */
+int nbh_memset8(void *dst, int byte, size_t nbytes, nbh_stream_t stream);
+
+/* ---- streams and events --------------------------------------------------- */
+
+/* cudadrv/driver.py:1244-1271 Context.create_stream (default flags: the stream
+ * synchronises with the legacy default stream), :1890-2017 Stream */
+int nbh_stream_create(nbh_stream_t *stream);
+int nbh_stream_destroy(nbh_stream_t stream);
+int nbh_stream_synchronize(nbh_stream_t stream);
+int nbh_stream_query(nbh_stream_t stream);
+/* cudadrv/driver.py:1273-1280 Context.create_event, :2037-2095 Event */
+int nbh_event_create(nbh_event_t *event, int timing);
+int nbh_event_destroy(nbh_event_t event);
+int nbh_event_record(nbh_event_t event, nbh_stream_t stream);
+int nbh_event_synchronize(nbh_event_t event);
+int nbh_event_query(nbh_event_t event);
+int nbh_stream_wait_event(nbh_stream_t stream, nbh_event_t event);
+int nbh_event_elapsed_ms(float *ms, nbh_event_t start, nbh_event_t stop);
+
+/* ---- reduction ------------------------------------------------------------ */
+
+/* Size of the scratch buffer nbh_reduce needs.  The caller allocates it in device
+ * memory, clears it to zero ONCE, and may then reuse it for any number of calls
+ * that do not overlap in time (one buffer per stream).  The library leaves it in
+ * the cleared state after every call. */
+size_t nbh_reduce_scratch_bytes(void);
+
+/* kernels/reduction.py:194-265 Reduce.__call__ together with the kernels it
+ * launches (:15-166).  Computes
+ *     out[0] = init (op) in[0] (op) in[1] (op) ... (op) in[n-1]
+ * for n >= 1 contiguous elements of `dtype` in device memory, in one launch and
+ * fully asynchronously on `stream`.  `init` points to one element of `dtype` in
+ * HOST memory (read before the call returns); `out` is one element in DEVICE
+ * memory (what `res[:1]` is in the reference).  The association order differs
+ * from the reference's (integer results are identical; floating-point sums agree
+ * within rounding, |err| <= 2 n eps sum|x|), and is the same on every run. */
+int nbh_reduce(int op, int dtype, const void *in, int64_t n, const void *init, void *out,
+               void *scratch, size_t scratch_bytes, nbh_stream_t stream);
+
+/* ---- transpose ------------------------------------------------------------ */
+
+/* kernels/transpose.py:10-65 transpose(a, b): out[j, i] = in[i, j] for a
+ * rows x cols input of items of `itemsize` bytes; all four strides are in bytes
+ * and arbitrary (views), any itemsize >= 1 (records).  The input and output
+ * regions must not overlap. */
+int nbh_transpose(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_stride0,
+                  int64_t in_stride1, int64_t out_stride0, int64_t out_stride1, int64_t itemsize,
+                  nbh_stream_t stream);
+
+/* ---- xoroshiro128+ -------------------------------------------------------- */
+
+/* random.py:241-282 init_xoroshiro128p_states (the sequential CPU jump chain plus
+ * the host-to-device copy): states[i] = jump^(subsequence_start + i)(seed state),
+ * computed on the device.  `states` is n records {uint64 s0; uint64 s1} (:47-50). */
+int nbh_xoro_init_states(void *states, int64_t n, uint64_t seed, uint64_t subsequence_start,
+                         nbh_stream_t stream);
+
+/* random.py:159-238 xoroshiro128p_{uniform,normal}_float{32,64} applied in bulk
+ * with the layout of the reference's test kernels (tests/cudapy/test_random.py
+ * :29-52): generator t draws `count` values into out[t*count + i], i ascending,
+ * and its state is advanced in place (by `count` steps for uniforms, 2*count for
+ * normals). */
+int nbh_xoro_uniform_f32(void *states, int64_t nstates, float *out, int64_t count, nbh_stream_t stream);
+int nbh_xoro_uniform_f64(void *states, int64_t nstates, double *out, int64_t count, nbh_stream_t stream);
+int nbh_xoro_normal_f32(void *states, int64_t nstates, float *out, int64_t count, nbh_stream_t stream);
+int nbh_xoro_normal_f64(void *states, int64_t nstates, double *out, int64_t count, nbh_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NBHIP_H */

@@ -1,0 +1,61 @@
+"""Ahead-of-time build of libnbhip.so (the HIP back end) for gfx950.
+
+    python -m numba_cuda_amd._build
+
+There is no JIT in this package: the kernels are compiled once, here, with hipcc.
+"""
+
+import os
+import shutil
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+SRC_DIR = os.path.join(PKG_DIR, "csrc")
+INCLUDE_DIR = os.path.join(os.path.dirname(PKG_DIR), "include")
+LIB_PATH = os.path.join(PKG_DIR, "libnbhip.so")
+
+SOURCES = ["runtime.hip", "reduce.hip", "transpose.hip", "xoroshiro.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # the reference compiles without fused multiply-add contraction
+    "-ffp-contract=off",
+    # keep the compiler from forming packed fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def find_hipcc():
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or install ROCm under /opt/rocm)")
+
+
+def build(verbose=False):
+    """Compile every HIP source into numba_cuda_amd/libnbhip.so; returns its path."""
+    cmd = [find_hipcc()] + HIPCC_FLAGS + ["-I", INCLUDE_DIR, "-I", SRC_DIR]
+    cmd += [os.path.join(SRC_DIR, s) for s in SOURCES]
+    tmp = LIB_PATH + ".tmp"
+    cmd += ["-o", tmp]
+    if verbose:
+        print(" ".join(cmd))
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # the host pass does not know the device-only target feature; that warning is noise
+    noise = ("packed-fp32-ops", "1 warning generated", "warnings generated")
+    out = "\n".join(l for l in proc.stdout.splitlines() if not any(k in l for k in noise))
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    if verbose and out.strip():
+        print(out)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

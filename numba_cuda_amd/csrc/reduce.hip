@@ -1,0 +1,298 @@
+// nbh_reduce: single-launch, deterministic tree reduction for gfx950 (wave64).
+//
+// Shape of the computation
+//   * the input is read once with 128-bit loads; the few elements in front of the
+//     first 16-byte boundary and behind the last whole vector are picked up by
+//     single lanes of workgroup 0
+//   * every workgroup (4 wavefronts) owns one contiguous slice of the vectors and
+//     walks it with UNROLL independent loads in flight per lane
+//   * lanes fold into per-lane accumulators, a wavefront folds with four DPP
+//     steps inside each row of 16 lanes plus three scalar combines of the four row
+//     totals, the workgroup folds its four wavefront totals through LDS
+//   * each workgroup publishes one partial; the workgroup that draws the last
+//     ticket folds the partials in index order, applies `init` and writes `out`.
+//     Which workgroup finishes does not change the association, so results are
+//     identical from run to run.
+//
+// HBM roofline: n * itemsize bytes are read once; nothing else of size is moved.
+#include "common.h"
+
+#include <limits>
+#include <type_traits>
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / 64;
+constexpr int kMaxGrid = 4096;
+constexpr size_t kHeaderBytes = 256;  // ticket counter, padded to its own cache lines
+constexpr size_t kScratchBytes = kHeaderBytes + sizeof(uint64_t) * kMaxGrid;
+constexpr int kGridPerCU = 8;
+constexpr int kUnroll = 4;
+
+// ---- operators -----------------------------------------------------------------
+struct OpAdd {
+    template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a + b; }
+};
+struct OpMul {
+    template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a * b; }
+};
+struct OpMax {
+    template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return b > a ? b : a; }
+};
+struct OpMin {
+    template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return b < a ? b : a; }
+};
+
+// Accumulator type.  Sums and products of integers are carried in an unsigned
+// type at least 32 bits wide: arithmetic modulo 2^32 / 2^64 truncates to the same
+// element value as arithmetic modulo 2^bits, and unsigned wrap-around is defined.
+// Comparisons keep the signedness of the element type.
+template <typename T, typename Op> struct AccOf {
+    static constexpr bool arith = std::is_same<Op, OpAdd>::value || std::is_same<Op, OpMul>::value;
+    using wide_int = typename std::conditional<
+        sizeof(T) == 8, typename std::conditional<arith || std::is_unsigned<T>::value, uint64_t, int64_t>::type,
+        typename std::conditional<arith || std::is_unsigned<T>::value, uint32_t, int32_t>::type>::type;
+    using type = typename std::conditional<std::is_floating_point<T>::value, T, wide_int>::type;
+};
+
+template <typename T, typename Op> __device__ __forceinline__ typename AccOf<T, Op>::type identity_of()
+{
+    using A = typename AccOf<T, Op>::type;
+    if constexpr (std::is_same<Op, OpAdd>::value)
+        return A(0);
+    else if constexpr (std::is_same<Op, OpMul>::value)
+        return A(1);
+    else if constexpr (std::is_same<Op, OpMax>::value)
+        return std::is_floating_point<T>::value ? A(-std::numeric_limits<T>::infinity())
+                                                : A(std::numeric_limits<T>::lowest());
+    else
+        return std::is_floating_point<T>::value ? A(std::numeric_limits<T>::infinity())
+                                                : A(std::numeric_limits<T>::max());
+}
+
+// ---- wavefront / workgroup folding -----------------------------------------------
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_move(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xF, 0xF, false);
+}
+
+template <typename A, int CTRL> __device__ __forceinline__ A dpp(A v)
+{
+    if constexpr (sizeof(A) == 4) {
+        uint32_t b = __builtin_bit_cast(uint32_t, v);
+        return __builtin_bit_cast(A, dpp_move<CTRL>(b));
+    } else {
+        uint64_t b = __builtin_bit_cast(uint64_t, v);
+        uint32_t lo = dpp_move<CTRL>((uint32_t)b);
+        uint32_t hi = dpp_move<CTRL>((uint32_t)(b >> 32));
+        return __builtin_bit_cast(A, ((uint64_t)hi << 32) | lo);
+    }
+}
+
+template <typename A> __device__ __forceinline__ A read_lane(A v, int lane)
+{
+    if constexpr (sizeof(A) == 4) {
+        uint32_t b = __builtin_bit_cast(uint32_t, v);
+        return __builtin_bit_cast(A, (uint32_t)__builtin_amdgcn_readlane((int)b, lane));
+    } else {
+        uint64_t b = __builtin_bit_cast(uint64_t, v);
+        uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, lane);
+        uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), lane);
+        return __builtin_bit_cast(A, ((uint64_t)hi << 32) | lo);
+    }
+}
+
+// Total of the 64 lanes, returned in every lane.
+template <typename A, typename Op> __device__ __forceinline__ A wave_fold(A v)
+{
+    v = Op::apply(v, dpp<A, 0xB1>(v));   // quad_perm [1,0,3,2]: lane ^ 1
+    v = Op::apply(v, dpp<A, 0x4E>(v));   // quad_perm [2,3,0,1]: lane ^ 2
+    v = Op::apply(v, dpp<A, 0x141>(v));  // row_half_mirror: the other quad of 8
+    v = Op::apply(v, dpp<A, 0x140>(v));  // row_mirror: the other half of 16
+    A r0 = read_lane(v, 0), r1 = read_lane(v, 16), r2 = read_lane(v, 32), r3 = read_lane(v, 48);
+    return Op::apply(Op::apply(r0, r1), Op::apply(r2, r3));
+}
+
+// Total of the workgroup, returned in every thread.  One LDS slot per wavefront.
+template <typename A, typename Op> __device__ __forceinline__ A block_fold(A v, A *lds)
+{
+    A w = wave_fold<A, Op>(v);
+    __syncthreads();  // slots may still be read from a previous fold
+    if ((threadIdx.x & 63) == 0)
+        lds[threadIdx.x >> 6] = w;
+    __syncthreads();
+    static_assert(kWaves == 4, "combine below assumes four wavefronts");
+    return Op::apply(Op::apply(lds[0], lds[1]), Op::apply(lds[2], lds[3]));
+}
+
+template <typename A> struct BitsOf {
+    using type = typename std::conditional<sizeof(A) == 8, uint64_t, uint32_t>::type;
+};
+
+// ---- the kernel ------------------------------------------------------------------
+template <typename T, typename Op>
+__global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in, int64_t n, int64_t head,
+                                                        int64_t nvec, T init, T *__restrict__ out,
+                                                        uint64_t *__restrict__ partials_raw,
+                                                        unsigned *__restrict__ ticket)
+{
+    using A = typename AccOf<T, Op>::type;
+    using Bits = typename BitsOf<A>::type;
+    constexpr int V = 16 / (int)sizeof(T);
+    typedef T VecT __attribute__((ext_vector_type(V)));
+
+    __shared__ A lds[kWaves];
+    __shared__ bool last_block;
+
+    const int tid = threadIdx.x;
+    A acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+        acc[j] = identity_of<T, Op>();
+
+    // contiguous slice of vectors owned by this workgroup
+    const VecT *__restrict__ vin = reinterpret_cast<const VecT *>(in + head);
+    const int64_t per = (nvec + gridDim.x - 1) / gridDim.x;
+    const int64_t begin = (int64_t)blockIdx.x * per;
+    int64_t end = begin + per;
+    if (end > nvec)
+        end = nvec;
+
+    int64_t i = begin + tid;
+    for (; i + (kUnroll - 1) * kBlock < end; i += kUnroll * kBlock) {
+        VecT v[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+            v[u] = __builtin_nontemporal_load(&vin[i + u * kBlock]);
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int j = 0; j < V; ++j)
+                acc[j] = Op::apply(acc[j], (A)v[u][j]);
+    }
+    for (; i < end; i += kBlock) {
+        VecT v = __builtin_nontemporal_load(&vin[i]);
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+            acc[j] = Op::apply(acc[j], (A)v[j]);
+    }
+
+    // elements outside the aligned body: fewer than 2 V, one per lane of workgroup 0
+    if (blockIdx.x == 0) {
+        const int64_t tail_begin = head + nvec * V;
+        if (tid < head)
+            acc[0] = Op::apply(acc[0], (A)in[tid]);
+        else if (tail_begin + (tid - head) < n)
+            acc[0] = Op::apply(acc[0], (A)in[tail_begin + (tid - head)]);
+    }
+
+    A mine = acc[0];
+#pragma unroll
+    for (int j = 1; j < V; ++j)
+        mine = Op::apply(mine, acc[j]);
+    A total = block_fold<A, Op>(mine, lds);
+
+    if (gridDim.x == 1) {
+        if (tid == 0)
+            out[0] = (T)Op::apply(total, (A)init);
+        return;
+    }
+
+    Bits *partials = reinterpret_cast<Bits *>(partials_raw);
+    if (tid == 0) {
+        __hip_atomic_store(&partials[blockIdx.x], __builtin_bit_cast(Bits, total), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+        // release the partial, acquire everybody else's
+        unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        last_block = (t == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (!last_block)
+        return;
+
+    A fin = identity_of<T, Op>();
+    for (int k = tid; k < (int)gridDim.x; k += kBlock) {
+        Bits b = __hip_atomic_load(&partials[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        fin = Op::apply(fin, __builtin_bit_cast(A, b));
+    }
+    fin = block_fold<A, Op>(fin, lds);
+    if (tid == 0) {
+        out[0] = (T)Op::apply(fin, (A)init);
+        // leave the scratch buffer as the caller handed it over
+        __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+template <typename T, typename Op>
+int launch(const void *in, int64_t n, const void *init, void *out, void *scratch, hipStream_t stream)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    const uintptr_t addr = (uintptr_t)in;
+    if (addr % sizeof(T) != 0 || ((uintptr_t)out) % sizeof(T) != 0)
+        return (int)hipErrorInvalidValue;
+    int64_t head = (int64_t)(((16 - (addr % 16)) % 16) / sizeof(T));
+    if (head > n)
+        head = n;
+    const int64_t nvec = (n - head) / V;
+
+    const int64_t per_block = (int64_t)kBlock * kUnroll;
+    int64_t grid = (nvec + per_block - 1) / per_block;
+    int64_t cap = (int64_t)nbh_cu_count() * kGridPerCU;
+    if (cap > kMaxGrid)
+        cap = kMaxGrid;
+    if (grid > cap)
+        grid = cap;
+    if (grid < 1)
+        grid = 1;
+
+    T init_value;
+    __builtin_memcpy(&init_value, init, sizeof(T));
+    unsigned *ticket = reinterpret_cast<unsigned *>(scratch);
+    uint64_t *partials = reinterpret_cast<uint64_t *>((char *)scratch + kHeaderBytes);
+    hipLaunchKernelGGL((reduce_kernel<T, Op>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
+                       (const T *)in, n, head, nvec, init_value, (T *)out, partials, ticket);
+    return nbh_launch_status();
+}
+
+template <typename T>
+int launch_op(int op, const void *in, int64_t n, const void *init, void *out, void *scratch, hipStream_t s)
+{
+    switch (op) {
+    case NBH_ADD: return launch<T, OpAdd>(in, n, init, out, scratch, s);
+    case NBH_MUL: return launch<T, OpMul>(in, n, init, out, scratch, s);
+    case NBH_MAX: return launch<T, OpMax>(in, n, init, out, scratch, s);
+    case NBH_MIN: return launch<T, OpMin>(in, n, init, out, scratch, s);
+    default: return (int)hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t nbh_reduce_scratch_bytes(void) { return kScratchBytes; }
+
+int nbh_reduce(int op, int dtype, const void *in, int64_t n, const void *init, void *out, void *scratch,
+               size_t scratch_bytes, nbh_stream_t stream)
+{
+    if (!in || !init || !out || !scratch || n < 1 || scratch_bytes < kScratchBytes ||
+        ((uintptr_t)scratch) % 8 != 0)
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = nbh_hip_stream(stream);
+    switch (dtype) {
+    case NBH_I8: return launch_op<int8_t>(op, in, n, init, out, scratch, s);
+    case NBH_I16: return launch_op<int16_t>(op, in, n, init, out, scratch, s);
+    case NBH_I32: return launch_op<int32_t>(op, in, n, init, out, scratch, s);
+    case NBH_I64: return launch_op<int64_t>(op, in, n, init, out, scratch, s);
+    case NBH_U8: return launch_op<uint8_t>(op, in, n, init, out, scratch, s);
+    case NBH_U16: return launch_op<uint16_t>(op, in, n, init, out, scratch, s);
+    case NBH_U32: return launch_op<uint32_t>(op, in, n, init, out, scratch, s);
+    case NBH_U64: return launch_op<uint64_t>(op, in, n, init, out, scratch, s);
+    case NBH_F32: return launch_op<float>(op, in, n, init, out, scratch, s);
+    case NBH_F64: return launch_op<double>(op, in, n, init, out, scratch, s);
+    default: return (int)hipErrorInvalidValue;
+    }
+}
+
+}  // extern "C"

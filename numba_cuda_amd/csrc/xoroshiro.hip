@@ -1,0 +1,363 @@
+// xoroshiro128+ (2016 constants 55/14/36) on gfx950: parallel state initialisation
+// and bulk uniform / normal draws.
+//
+// State initialisation.  The reference builds states[i] = jump^i(states[0]) as one
+// sequential chain on the CPU.  `next` is linear over GF(2), so `jump` (2^64 steps)
+// is a 128x128 bit matrix J; the host tabulates J^(2^k), k = 0..63, once per
+// process, and lane l of a wavefront computes J^(base+l) * s by binary expansion of
+// the exponent (bits >= 6 are uniform across the wavefront), then keeps stepping by
+// J^64 so that each step of the wavefront writes 64 consecutive states (1 KiB).
+//
+// Draws.  Each lane owns one generator whose 128-bit state stays in registers.
+// The reference's layout out[t*count + i] gives every lane its own run of `count`
+// values, so values are parked in LDS for a round and written back with the run
+// index fastest: every store instruction of a wavefront covers whole 128-byte lines.
+//
+// HBM roofline: out bytes written + 2 * 16 bytes of state per generator.
+#include "common.h"
+
+#include <mutex>
+
+namespace {
+
+// ---- host side: the jump matrices ---------------------------------------------
+
+struct U128 {
+    uint64_t s0, s1;
+};
+
+inline uint64_t rotl_h(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+
+inline void next_h(U128 &s)
+{
+    uint64_t a = s.s0, b = s.s1 ^ s.s0;
+    s.s0 = rotl_h(a, 55) ^ b ^ (b << 14);
+    s.s1 = rotl_h(b, 36);
+}
+
+inline U128 jump_h(U128 s)
+{
+    const uint64_t poly[2] = {0xBEAC0467EBA5FACBull, 0xD86B048B86AA9922ull};
+    U128 acc = {0, 0};
+    for (int w = 0; w < 2; ++w)
+        for (int b = 0; b < 64; ++b) {
+            if ((poly[w] >> b) & 1) {
+                acc.s0 ^= s.s0;
+                acc.s1 ^= s.s1;
+            }
+            next_h(s);
+        }
+    return acc;
+}
+
+constexpr int kPowers = 64;
+// table[k][c] = column c of J^(2^k): the image of the state with only bit c set
+// (bits 0..63 live in s0, bits 64..127 in s1).
+struct JumpTable {
+    U128 col[kPowers][128];
+};
+
+inline U128 apply_h(const U128 *m, U128 v)
+{
+    U128 r = {0, 0};
+    for (int b = 0; b < 64; ++b) {
+        if ((v.s0 >> b) & 1) {
+            r.s0 ^= m[b].s0;
+            r.s1 ^= m[b].s1;
+        }
+        if ((v.s1 >> b) & 1) {
+            r.s0 ^= m[64 + b].s0;
+            r.s1 ^= m[64 + b].s1;
+        }
+    }
+    return r;
+}
+
+const JumpTable &jump_table()
+{
+    static JumpTable *table = nullptr;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        JumpTable *t = new JumpTable;
+        for (int c = 0; c < 128; ++c) {
+            U128 e = {c < 64 ? (1ull << c) : 0, c < 64 ? 0 : (1ull << (c - 64))};
+            t->col[0][c] = jump_h(e);
+        }
+        for (int k = 1; k < kPowers; ++k)  // square: column c of M*M is M applied to column c of M
+            for (int c = 0; c < 128; ++c)
+                t->col[k][c] = apply_h(t->col[k - 1], t->col[k - 1][c]);
+        table = t;
+    });
+    return *table;
+}
+
+// Device copy of the table, one per device, made on first use and kept for the
+// life of the process (128 KiB).
+int device_table(const U128 **out)
+{
+    constexpr int kMaxDev = 64;
+    static const U128 *cache[kMaxDev] = {};
+    static std::mutex mu;
+    int dev = 0;
+    NBH_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDev)
+        return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!cache[dev]) {
+        const JumpTable &t = jump_table();
+        void *d = nullptr;
+        NBH_TRY(hipMalloc(&d, sizeof(JumpTable)));
+        hipError_t e = hipMemcpy(d, &t, sizeof(JumpTable), hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(d);
+            return (int)e;
+        }
+        cache[dev] = (const U128 *)d;
+    }
+    *out = cache[dev];
+    return 0;
+}
+
+// ---- device side ------------------------------------------------------------------
+
+__device__ __forceinline__ uint64_t rotl_d(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+
+__device__ __forceinline__ uint64_t next_d(uint64_t &s0, uint64_t &s1)
+{
+    const uint64_t r = s0 + s1;
+    const uint64_t t = s1 ^ s0;
+    s0 = rotl_d(s0, 55) ^ t ^ (t << 14);
+    s1 = rotl_d(t, 36);
+    return r;
+}
+
+// r = M * (s0, s1) over GF(2); m is wavefront-uniform, so its columns come in
+// through scalar loads.
+__device__ __forceinline__ void apply_d(const U128 *__restrict__ m, uint64_t &s0, uint64_t &s1)
+{
+    uint64_t r0 = 0, r1 = 0;
+#pragma unroll 8
+    for (int b = 0; b < 64; ++b) {
+        const uint64_t m0 = 0 - ((s0 >> b) & 1);
+        const uint64_t m1 = 0 - ((s1 >> b) & 1);
+        r0 ^= (m[b].s0 & m0) ^ (m[64 + b].s0 & m1);
+        r1 ^= (m[b].s1 & m0) ^ (m[64 + b].s1 & m1);
+    }
+    s0 = r0;
+    s1 = r1;
+}
+
+constexpr int kInitBlock = 256;
+constexpr int kInitSteps = 64;  // consecutive 64-state groups produced by one wavefront
+
+__global__ __launch_bounds__(kInitBlock) void init_states_kernel(uint64_t *__restrict__ states, int64_t n,
+                                                                 uint64_t b0, uint64_t b1,
+                                                                 const U128 *__restrict__ table)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kInitBlock / 64) + (threadIdx.x >> 6);
+    const int64_t first = wave * (64 * kInitSteps);  // first state index of this wavefront
+    if (first >= n)
+        return;
+    uint64_t s0 = b0, s1 = b1;
+    // J^first: every bit of `first` below 6 is zero; the rest is uniform
+    const uint64_t hi = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 6)) |
+                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 38)) << 32);
+    for (int k = 6; k < kPowers; ++k)
+        if ((hi >> (k - 6)) & 1)
+            apply_d(table + (size_t)k * 128, s0, s1);
+    // J^lane
+    for (int k = 0; k < 6; ++k)
+        if ((lane >> k) & 1)
+            apply_d(table + (size_t)k * 128, s0, s1);
+    const U128 *__restrict__ step = table + (size_t)6 * 128;  // J^64
+    for (int g = 0; g < kInitSteps; ++g) {
+        const int64_t idx = first + (int64_t)g * 64 + lane;
+        if (first + (int64_t)g * 64 >= n)
+            break;
+        if (idx < n) {
+            typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+            u64x2 v = {s0, s1};
+            *reinterpret_cast<u64x2 *>(states + 2 * idx) = v;
+        }
+        if (g + 1 < kInitSteps)
+            apply_d(step, s0, s1);
+    }
+}
+
+// ---- draws -------------------------------------------------------------------------
+
+struct UniformF32 {
+    using value_type = float;
+    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1)
+    {
+        // one exact product in double, one rounding to float
+        return (float)((double)(next_d(s0, s1) >> 11) * (1.0 / 9007199254740992.0));
+    }
+};
+struct UniformF64 {
+    using value_type = double;
+    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1)
+    {
+        return (double)(next_d(s0, s1) >> 11) * (1.0 / 9007199254740992.0);
+    }
+};
+// Box-Muller, cosine branch.  The float32 variant works in float32 throughout;
+// log and cos are evaluated in double and rounded once, which is the closest
+// available stand-in for correctly rounded float32 routines.
+struct NormalF32 {
+    using value_type = float;
+    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1)
+    {
+        const float u1 = UniformF32::draw(s0, s1);
+        const float u2 = UniformF32::draw(s0, s1);
+        const float two_pi = 6.283185307179586f;
+        const float lg = (float)log((double)u1);
+        const float r = sqrtf(-2.0f * lg);
+        const float c = (float)cos((double)(two_pi * u2));
+        return r * c;
+    }
+};
+// The float64 variant still draws float32 uniforms and takes the logarithm of a
+// float32 (so its result is a float32); the square root and cosine are float64.
+struct NormalF64 {
+    using value_type = double;
+    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1)
+    {
+        const float u1 = UniformF32::draw(s0, s1);
+        const float u2 = UniformF32::draw(s0, s1);
+        const double two_pi = 6.283185307179586;
+        const float lg = (float)log((double)u1);
+        const double r = sqrt(-2.0 * (double)lg);
+        const double c = cos(two_pi * (double)u2);
+        return r * c;
+    }
+};
+
+constexpr int kFillBlock = 256;
+
+template <typename Gen>
+__global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__ states, int64_t n,
+                                                          typename Gen::value_type *__restrict__ out,
+                                                          int64_t count)
+{
+    using VT = typename Gen::value_type;
+    constexpr int ROUND = 128 / (int)sizeof(VT);  // one 128-byte line per generator per round
+    __shared__ VT park[kFillBlock][ROUND + 1];
+
+    const int tid = threadIdx.x;
+    const int64_t t0 = (int64_t)blockIdx.x * kFillBlock;  // first generator of this workgroup
+    const int64_t t = t0 + tid;
+    const bool live = t < n;
+    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+    uint64_t s0 = 0, s1 = 0;
+    if (live) {
+        u64x2 v = *reinterpret_cast<const u64x2 *>(states + 2 * t);
+        s0 = v.x;
+        s1 = v.y;
+    }
+    int64_t lanes_here = n - t0;  // generators this workgroup really has
+    if (lanes_here > kFillBlock)
+        lanes_here = kFillBlock;
+    VT *__restrict__ base = out + t0 * count;
+
+    for (int64_t i0 = 0; i0 < count; i0 += ROUND) {
+        const int m = (int)((count - i0 < ROUND) ? (count - i0) : ROUND);
+        if (live)
+            for (int j = 0; j < m; ++j)
+                park[tid][j] = Gen::draw(s0, s1);
+        __syncthreads();
+        if (m == ROUND) {
+#pragma unroll 4
+            for (int f = tid; f < kFillBlock * ROUND; f += kFillBlock) {
+                const int l = f / ROUND, j = f % ROUND;
+                if (l < lanes_here)
+                    base[(int64_t)l * count + i0 + j] = park[l][j];
+            }
+        } else {
+            for (int f = tid; f < kFillBlock * m; f += kFillBlock) {
+                const int l = f / m, j = f % m;
+                if (l < lanes_here)
+                    base[(int64_t)l * count + i0 + j] = park[l][j];
+            }
+        }
+        __syncthreads();
+    }
+    if (live) {
+        u64x2 v = {s0, s1};
+        *reinterpret_cast<u64x2 *>(states + 2 * t) = v;
+    }
+}
+
+template <typename Gen>
+int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t stream)
+{
+    if (n < 0 || count < 0)
+        return (int)hipErrorInvalidValue;
+    if (n == 0 || count == 0)
+        return 0;
+    if (!states || !out || ((uintptr_t)states) % 16 != 0 ||
+        ((uintptr_t)out) % sizeof(typename Gen::value_type) != 0)
+        return (int)hipErrorInvalidValue;
+    const int64_t grid = (n + kFillBlock - 1) / kFillBlock;
+    if (grid > 0x7fffffffLL)
+        return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((fill_kernel<Gen>), dim3((unsigned)grid), dim3(kFillBlock), 0, nbh_hip_stream(stream),
+                       (uint64_t *)states, n, (typename Gen::value_type *)out, count);
+    return nbh_launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int nbh_xoro_init_states(void *states, int64_t n, uint64_t seed, uint64_t subsequence_start, nbh_stream_t stream)
+{
+    if (n < 0)
+        return (int)hipErrorInvalidValue;
+    if (n == 0)
+        return 0;
+    if (!states || ((uintptr_t)states) % 16 != 0)
+        return (int)hipErrorInvalidValue;
+    // SplitMix64 step; the same word seeds both halves
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    U128 base = {z, z};
+    // advance to the first subsequence on the host: at most 64 matrix products
+    const JumpTable &t = jump_table();
+    for (int k = 0; k < kPowers; ++k)
+        if ((subsequence_start >> k) & 1)
+            base = apply_h(t.col[k], base);
+    const U128 *dtable = nullptr;
+    int rc = device_table(&dtable);
+    if (rc)
+        return rc;
+    const int64_t per_block = (int64_t)(kInitBlock / 64) * 64 * kInitSteps;
+    const int64_t grid = (n + per_block - 1) / per_block;
+    if (grid > 0x7fffffffLL)
+        return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(init_states_kernel, dim3((unsigned)grid), dim3(kInitBlock), 0, nbh_hip_stream(stream),
+                       (uint64_t *)states, n, base.s0, base.s1, dtable);
+    return nbh_launch_status();
+}
+
+int nbh_xoro_uniform_f32(void *states, int64_t nstates, float *out, int64_t count, nbh_stream_t stream)
+{
+    return launch_fill<UniformF32>(states, nstates, out, count, stream);
+}
+int nbh_xoro_uniform_f64(void *states, int64_t nstates, double *out, int64_t count, nbh_stream_t stream)
+{
+    return launch_fill<UniformF64>(states, nstates, out, count, stream);
+}
+int nbh_xoro_normal_f32(void *states, int64_t nstates, float *out, int64_t count, nbh_stream_t stream)
+{
+    return launch_fill<NormalF32>(states, nstates, out, count, stream);
+}
+int nbh_xoro_normal_f64(void *states, int64_t nstates, double *out, int64_t count, nbh_stream_t stream)
+{
+    return launch_fill<NormalF64>(states, nstates, out, count, stream);
+}
+
+}  // extern "C"
