@@ -1,0 +1,214 @@
+"""`Reduce`: full reduction of a 1-d array with a binary operator.
+
+Drop-in for numba_cuda/numba/cuda/kernels/reduction.py:169-265.  The reference
+JIT-compiles the Python functor into a three-launch tree reduction; here the
+functor is *recognised* as one of the four operators that have hand-written HIP
+kernels (a + b, a * b, max(a, b), min(a, b)) and a single launch of
+nbh_reduce does the work.  Anything else raises NotImplementedError - there is
+no slower path to fall back to.
+"""
+
+import operator
+
+import numpy as np
+
+from numba_cuda_amd import _lib
+from numba_cuda_amd.cudadrv import devicearray, devices
+from numba_cuda_amd.cudadrv import driver as _driver
+
+
+class _Sym:
+    """Operand stand-in that records which operator the functor applies."""
+
+    def __init__(self, name, log):
+        self.name, self.log = name, log
+
+    def _binary(self, opname, other, swapped=False):
+        if not isinstance(other, _Sym):
+            raise _Unrecognised("operand mixed with a constant")
+        lhs, rhs = (other, self) if swapped else (self, other)
+        self.log.append((opname, lhs.name, rhs.name))
+        return _Sym("(%s %s %s)" % (lhs.name, opname, rhs.name), self.log)
+
+    def __add__(self, o):
+        return self._binary("add", o)
+
+    def __radd__(self, o):
+        return self._binary("add", o, True)
+
+    def __mul__(self, o):
+        return self._binary("mul", o)
+
+    def __rmul__(self, o):
+        return self._binary("mul", o, True)
+
+    def _compare(self, opname, other):
+        if not isinstance(other, _Sym):
+            raise _Unrecognised("operand compared with a constant")
+        return _Cond(opname, self.name, other.name, self.log)
+
+    def __gt__(self, o):
+        return self._compare("gt", o)
+
+    def __lt__(self, o):
+        return self._compare("lt", o)
+
+    def __ge__(self, o):
+        return self._compare("ge", o)
+
+    def __le__(self, o):
+        return self._compare("le", o)
+
+    def __bool__(self):
+        raise _Unrecognised("truth value of an operand")
+
+
+class _Cond:
+    """Result of comparing two stand-ins; its truth value is scripted."""
+
+    def __init__(self, opname, lhs, rhs, log):
+        self.key = (opname, lhs, rhs)
+        self.log = log
+
+    def __bool__(self):
+        self.log.append(("cmp",) + self.key)
+        return self.log.answer
+
+
+class _Log(list):
+    answer = True
+
+
+class _Unrecognised(Exception):
+    pass
+
+
+_DIRECT = {operator.add: "add", operator.mul: "mul", max: "max", min: "min",
+           np.add: "add", np.multiply: "mul"}
+
+
+def _trace(functor, answer):
+    log = _Log()
+    log.answer = answer
+    out = functor(_Sym("a", log), _Sym("b", log))
+    if not isinstance(out, _Sym):
+        raise _Unrecognised("functor did not return one of its operands or their sum/product")
+    return out.name, list(log)
+
+
+def classify_functor(functor):
+    """-> "add" | "mul" | "max" | "min", or NotImplementedError.
+
+    The functor is run on two recording stand-ins.  `a + b` / `a * b` show up as
+    one arithmetic event.  `max(a, b)` / `min(a, b)` and the equivalent
+    conditional expressions show up as one comparison whose scripted outcome
+    decides which operand comes back; running with both outcomes tells max from
+    min.  The verdict is then confirmed on real numbers."""
+    try:
+        if functor in _DIRECT:
+            return _DIRECT[functor]
+    except TypeError:
+        pass
+    verdict = None
+    try:
+        name_t, log_t = _trace(functor, True)
+        name_f, log_f = _trace(functor, False)
+        if len(log_t) == 1 and log_t == log_f and log_t[0][0] in ("add", "mul"):
+            if {log_t[0][1], log_t[0][2]} == {"a", "b"}:
+                verdict = log_t[0][0]
+        elif (len(log_t) == 1 and len(log_f) == 1 and log_t[0][0] == "cmp" and log_t == log_f
+              and {name_t, name_f} == {"a", "b"}):
+            _, cmp_op, lhs, rhs = log_t[0]
+            if {lhs, rhs} == {"a", "b"}:
+                # when "lhs <cmp_op> rhs" holds the functor returns name_t
+                greater_wins = (cmp_op in ("gt", "ge")) == (name_t == lhs)
+                verdict = "max" if greater_wins else "min"
+    except _Unrecognised:
+        verdict = None
+    except Exception:
+        verdict = None
+    if verdict is not None:
+        probes = {"add": 8, "mul": 15, "max": 5, "min": 3}
+        try:
+            ok = functor(3, 5) == probes[verdict] and functor(5, 3) == probes[verdict]
+        except Exception:
+            ok = False
+        if ok:
+            return verdict
+    raise NotImplementedError(
+        "Reduce supports the binary operators a + b, a * b, max(a, b) and min(a, b); "
+        "%r was not recognised as one of them" % (functor,))
+
+
+class Reduce:
+    """Reduction object for a binary function; the recognised operator is cached
+    in the object and per functor."""
+
+    _cache = {}
+
+    def __init__(self, functor):
+        """`functor`: the binary operation, e.g. ``lambda a, b: a + b``."""
+        self._functor = functor
+        try:
+            self._op = self._cache[functor]
+        except (KeyError, TypeError):
+            self._op = classify_functor(functor)
+            try:
+                self._cache[functor] = self._op
+            except TypeError:
+                pass
+
+    def __call__(self, arr, size=None, res=None, init=0, stream=0):
+        """Full reduction of `arr`.
+
+        arr    : 1-d host or device array
+        size   : reduce only the first `size` items
+        res    : device array; the result goes into its first item and nothing is
+                 copied to the host (the call is then fully asynchronous)
+        init   : initial value, converted to arr.dtype
+        stream : stream to work on (0: the default stream)
+        Returns the result as a NumPy scalar, or None when `res` is given.
+        """
+        if arr.ndim != 1:
+            raise TypeError("only support 1D array")
+        if size is not None:
+            arr = arr[:size]
+        init = arr.dtype.type(init)
+        if arr.size < 1:
+            return init          # `res` is left untouched, as in the reference
+
+        code = _lib.DTYPE_CODES.get(arr.dtype.name)
+        if code is None or not arr.dtype.isnative:
+            raise NotImplementedError("Reduce does not support dtype %s" % arr.dtype)
+
+        ctx = devices.get_context()
+        if not _driver.is_device_memory(arr):
+            # host input: implicit transfer, as a kernel argument would get
+            arr, _ = devicearray.auto_device(arr, stream=stream)
+        if arr.strides[0] != arr.dtype.itemsize:
+            raise NotImplementedError("Reduce needs a unit-stride array; got strides %s" % (arr.strides,))
+
+        hstream = _driver._stream_handle(stream)
+        scratch, slot = ctx.reduce_scratch(hstream)
+        if res is not None:
+            if res.dtype != arr.dtype:
+                raise TypeError("res has dtype %s, expected %s" % (res.dtype, arr.dtype))
+            out_ptr = res.device_ctypes_pointer.value
+        else:
+            out_ptr = slot      # per-stream result slot: no allocation per call
+        init_buf = np.array([init], dtype=arr.dtype)
+        _driver.driver.nbh_reduce(_lib.OP_CODES[self._op], code, arr.device_ctypes_pointer.value,
+                                  arr.size, init_buf.ctypes.data, out_ptr,
+                                  scratch.device_ctypes_pointer.value, ctx.reduce_scratch_bytes,
+                                  hstream or None)
+        if res is not None:
+            return None
+        # the value is wanted on the host now: wait for the stream, then fetch it
+        if hstream:
+            _driver.driver.nbh_stream_synchronize(hstream)
+        host = np.empty(1, dtype=arr.dtype)
+        _driver.driver.nbh_memcpy_d2h(host.ctypes.data, out_ptr, arr.dtype.itemsize, None)
+        return host[0]
+
+
+reduce = Reduce

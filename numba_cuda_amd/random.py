@@ -1,0 +1,201 @@
+"""xoroshiro128+ random numbers (drop-in for numba_cuda/numba/cuda/random.py).
+
+Differences in mechanism, not in results:
+  * init_xoroshiro128p_states builds the states ON THE DEVICE (GF(2) jump
+    matrices) instead of as a sequential CPU chain followed by an upload; the
+    states are bit-identical to the reference's (random.py:241-282)
+  * the reference offers per-thread device functions for use inside JIT kernels;
+    there is no kernel language here, so draws are bulk operations:
+    `xoroshiro128p_fill(states, out, count, distribution)` produces, for every
+    generator t, `count` values into out[t*count + i] - the layout of the
+    reference's own test kernels (tests/cudapy/test_random.py:29-52)
+  * the scalar functions `xoroshiro128p_next(states, index)` etc. keep their
+    reference meaning on HOST state arrays (the reference's functions are also
+    CPU-callable); device arrays are refused with a pointer to the bulk call.
+"""
+
+import math
+
+import numpy as np
+
+from numba_cuda_amd.cudadrv import devicearray, devices
+from numba_cuda_amd.cudadrv import driver as _driver
+from numba_cuda_amd import api as _api
+
+xoroshiro128p_dtype = np.dtype([("s0", np.uint64), ("s1", np.uint64)], align=True)
+
+UNIFORM = 1
+NORMAL = 2
+
+_M64 = (1 << 64) - 1
+
+
+# ---- bulk device operations -----------------------------------------------------------
+
+def _check_states(states):
+    if states.ndim != 1 or states.dtype.itemsize != 16:
+        raise TypeError("states must be a 1D array of xoroshiro128p_dtype")
+    if not _driver.is_device_memory(states):
+        raise TypeError("states must be a device array (see create_xoroshiro128p_states)")
+    if states.size and states.strides[0] != 16:
+        raise ValueError("states must have unit stride")
+
+
+@devices.require_context
+def init_xoroshiro128p_states(states, seed, subsequence_start=0, stream=0):
+    """Initialise `states` so that states[i] is the generator seeded with `seed`
+    advanced by (subsequence_start + i) * 2**64 steps: independent subsequences
+    as long as no generator draws more than 2**64 numbers.
+
+    states : 1D DeviceNDArray of xoroshiro128p_dtype
+    seed, subsequence_start : reduced modulo 2**64
+    """
+    _check_states(states)
+    _driver.driver.nbh_xoro_init_states(states.device_ctypes_pointer.value, states.size,
+                                        int(seed) & _M64, int(subsequence_start) & _M64,
+                                        _driver._stream_handle(stream) or None)
+
+
+@devices.require_context
+def create_xoroshiro128p_states(n, seed, subsequence_start=0, stream=0):
+    """New device array of `n` initialised generator states."""
+    states = _api.device_array(n, dtype=xoroshiro128p_dtype, stream=stream)
+    init_xoroshiro128p_states(states, seed, subsequence_start, stream)
+    return states
+
+
+_FILL = {
+    (UNIFORM, "float32"): "nbh_xoro_uniform_f32",
+    (UNIFORM, "float64"): "nbh_xoro_uniform_f64",
+    (NORMAL, "float32"): "nbh_xoro_normal_f32",
+    (NORMAL, "float64"): "nbh_xoro_normal_f64",
+}
+
+
+@devices.require_context
+def xoroshiro128p_fill(states, out, count=None, distribution=UNIFORM, stream=0):
+    """Every generator t draws `count` values of out.dtype into
+    out[t*count + i], i = 0..count-1, and its state advances in place (by `count`
+    steps for UNIFORM, 2*count for NORMAL - Box-Muller uses two draws per value).
+
+    out          : 1D device array of float32 or float64 with at least
+                   len(states)*count items; `count` defaults to out.size // len(states)
+    distribution : UNIFORM -> [0, 1)  (float32 values may round up to exactly 1.0,
+                   as in the reference), NORMAL -> mean 0, sigma 1
+    """
+    _check_states(states)
+    if not _driver.is_device_memory(out):
+        raise TypeError("out must be a device array")
+    if out.ndim != 1 or (out.size and out.strides[0] != out.dtype.itemsize):
+        raise ValueError("out must be a 1D unit-stride array")
+    n = states.size
+    if count is None:
+        count = out.size // n if n else 0
+    count = int(count)
+    if count < 0 or n * count > out.size:
+        raise ValueError("out has %d items, need %d generators x %d draws" % (out.size, n, count))
+    fn = _FILL.get((distribution, out.dtype.name))
+    if fn is None:
+        raise TypeError("unsupported distribution/dtype: %r / %s" % (distribution, out.dtype))
+    getattr(_driver.driver, fn)(states.device_ctypes_pointer.value, n, out.device_ctypes_pointer.value,
+                                count, _driver._stream_handle(stream) or None)
+    return out
+
+
+def xoroshiro128p_fill_uniform(states, out, count=None, stream=0):
+    return xoroshiro128p_fill(states, out, count, UNIFORM, stream)
+
+
+def xoroshiro128p_fill_normal(states, out, count=None, stream=0):
+    return xoroshiro128p_fill(states, out, count, NORMAL, stream)
+
+
+# ---- scalar functions on host state arrays (reference semantics, random.py:62-238) ----
+
+def _host_states(states):
+    if _driver.is_device_memory(states):
+        raise TypeError("per-generator draws need a host array of states; on the device use "
+                        "xoroshiro128p_fill(states, out, count, distribution)")
+    return states
+
+
+def init_xoroshiro128p_state(states, index, seed):
+    """SplitMix64 step of `seed`; the same word goes into both halves."""
+    states = _host_states(states)
+    z = (int(seed) + 0x9E3779B97F4A7C15) & _M64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    z ^= z >> 31
+    states[int(index)]["s0"] = z
+    states[int(index)]["s1"] = z
+
+
+def rotl(x, k):
+    x = int(x) & _M64
+    return ((x << k) & _M64) | (x >> (64 - k))
+
+
+def xoroshiro128p_next(states, index):
+    """Next uint64 of generator `index`; advances it."""
+    states = _host_states(states)
+    index = int(index)
+    s0 = int(states[index]["s0"])
+    s1 = int(states[index]["s1"])
+    result = (s0 + s1) & _M64
+    s1 ^= s0
+    states[index]["s0"] = rotl(s0, 55) ^ s1 ^ ((s1 << 14) & _M64)
+    states[index]["s1"] = rotl(s1, 36)
+    return np.uint64(result)
+
+
+def xoroshiro128p_jump(states, index):
+    """Advance generator `index` by 2**64 steps."""
+    states = _host_states(states)
+    index = int(index)
+    s0 = s1 = 0
+    for word in (0xBEAC0467EBA5FACB, 0xD86B048B86AA9922):
+        for b in range(64):
+            if (word >> b) & 1:
+                s0 ^= int(states[index]["s0"])
+                s1 ^= int(states[index]["s1"])
+            xoroshiro128p_next(states, index)
+    states[index]["s0"] = s0
+    states[index]["s1"] = s1
+
+
+def uint64_to_unit_float64(x):
+    return np.float64((int(x) >> 11) * (1.0 / (1 << 53)))
+
+
+def uint64_to_unit_float32(x):
+    return np.float32(uint64_to_unit_float64(x))
+
+
+def xoroshiro128p_uniform_float32(states, index):
+    return uint64_to_unit_float32(xoroshiro128p_next(states, index))
+
+
+def xoroshiro128p_uniform_float64(states, index):
+    return uint64_to_unit_float64(xoroshiro128p_next(states, index))
+
+
+TWO_PI_FLOAT32 = np.float32(2 * math.pi)
+TWO_PI_FLOAT64 = np.float64(2 * math.pi)
+
+
+def xoroshiro128p_normal_float32(states, index):
+    """Box-Muller (cosine branch) in float32; uses two draws."""
+    u1 = xoroshiro128p_uniform_float32(states, index)
+    u2 = xoroshiro128p_uniform_float32(states, index)
+    with np.errstate(divide="ignore"):
+        r = np.sqrt(-np.float32(2.0) * np.log(u1))
+    return np.float32(r * np.cos(TWO_PI_FLOAT32 * u2))
+
+
+def xoroshiro128p_normal_float64(states, index):
+    """Box-Muller (cosine branch); float32 uniforms and logarithm, float64 rest."""
+    u1 = xoroshiro128p_uniform_float32(states, index)
+    u2 = xoroshiro128p_uniform_float32(states, index)
+    with np.errstate(divide="ignore"):
+        r = np.sqrt(-np.float64(2.0) * np.float64(np.log(u1)))
+    return np.float64(r * np.cos(TWO_PI_FLOAT64 * np.float64(u2)))

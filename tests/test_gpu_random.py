@@ -1,0 +1,177 @@
+"""Parity of the xoroshiro128+ device path with the oracle: states and uniform
+bits exact; Box-Muller normals within 2 ulp of the correctly rounded restatement
+(their bit-level parity with the reference's libdevice is unpinned: no file of
+the reference records those bits)."""
+
+import math
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import numba_cuda_amd as cuda
+from numba_cuda_amd import random as nrandom
+from oracle import cref
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def test_create_distinct_states():
+    # numba_cuda/numba/cuda/tests/cudapy/test_random.py:57-60
+    s = cuda.random.create_xoroshiro128p_states(10, seed=1).copy_to_host()
+    assert s.dtype == nrandom.xoroshiro128p_dtype
+    assert len(np.unique(s)) == 10
+
+
+def test_create_subsequence_start():
+    # test_random.py:62-72
+    s1 = cuda.random.create_xoroshiro128p_states(10, seed=1).copy_to_host()
+    s2 = cuda.random.create_xoroshiro128p_states(10, seed=1, subsequence_start=3).copy_to_host()
+    np.testing.assert_array_equal(s1[3:], s2[:-3])
+
+
+def test_create_stream():
+    stream = cuda.stream()
+    s = cuda.random.create_xoroshiro128p_states(10, seed=1, stream=stream)
+    stream.synchronize()
+    assert len(np.unique(s.copy_to_host())) == 10
+
+
+@pytest.mark.parametrize("n,seed,start", [(1, 0, 0), (10, 1, 0), (63, 1, 1), (64, 42, 0), (65, 42, 5),
+                                          (4095, 7, 2), (4097, 2**64 - 1, 0), (16385, -3, 9),
+                                          (70001, 42, 0), (300000, 12345678901234567890, 17)])
+def test_states_bit_exact_against_sequential_chain(n, seed, start):
+    _say("states", n, seed, start)
+    got = cuda.random.create_xoroshiro128p_states(n, seed=seed, subsequence_start=start).copy_to_host()
+    np.testing.assert_array_equal(got, cref.init_states(n, seed, start))
+
+
+def test_huge_subsequence_start_is_consistent():
+    """2^40+3 and 2^64-1 jumps cannot be walked sequentially; the chain property
+    states[i+1] == jump(states[i]) and the shift property still pin them."""
+    for start in (2**40 + 3, 2**64 - 1):
+        got = cuda.random.create_xoroshiro128p_states(300, seed=9, subsequence_start=start).copy_to_host()
+        st = np.array([got[0]["s0"], got[0]["s1"]], np.uint64)
+        for i in range(1, 300):
+            cref.jump(st)
+            assert (got[i]["s0"], got[i]["s1"]) == (st[0], st[1])
+    a = cuda.random.create_xoroshiro128p_states(5, seed=9, subsequence_start=2**40).copy_to_host()
+    b = cuda.random.create_xoroshiro128p_states(5, seed=9, subsequence_start=2**40 + 2).copy_to_host()
+    np.testing.assert_array_equal(a[2:], b[:-2])
+
+
+def _ulps(got, want):
+    fin = np.isfinite(want)
+    assert np.array_equal(got[~fin], want[~fin], equal_nan=True)
+    return np.abs(got[fin].astype(np.float64) - want[fin].astype(np.float64)) / \
+        np.spacing(np.abs(want[fin])).astype(np.float64)
+
+
+@pytest.mark.parametrize("n", [1, 64, 257, 5000])
+@pytest.mark.parametrize("kind,count", [("uniform_f32", 64), ("uniform_f32", 1), ("uniform_f32", 33),
+                                        ("uniform_f64", 7), ("uniform_f64", 40),
+                                        ("normal_f32", 33), ("normal_f64", 16)])
+def test_fill_against_oracle(n, kind, count):
+    _say("fill", kind, n, count)
+    host_states = cref.init_states(n, 42, 5)
+    states = cuda.to_device(host_states)
+    dtype = np.float32 if kind.endswith("f32") else np.float64
+    out = cuda.device_array(n * count, dtype=dtype)
+    dist = nrandom.UNIFORM if kind.startswith("uniform") else nrandom.NORMAL
+    nrandom.xoroshiro128p_fill(states, out, count, dist)
+    want, want_states = cref.fill(host_states, count, kind)
+    got = out.copy_to_host()
+    np.testing.assert_array_equal(states.copy_to_host(), want_states)
+    if dist == nrandom.UNIFORM:
+        assert got.tobytes() == want.tobytes()
+    else:
+        assert _ulps(got, want).max() <= 2.0      # tolerance: 2 ulp
+
+
+def test_reference_statistics():
+    # test_random.py:82-113
+    for dtype in (np.float32, np.float64):
+        states = cuda.random.create_xoroshiro128p_states(64, seed=1)
+        out = cuda.device_array(64 * 32, dtype=dtype)
+        u = nrandom.xoroshiro128p_fill(states, out, 32, nrandom.UNIFORM).copy_to_host()
+        assert abs(u.min()) < 1e-3 and abs(u.max() - 1.0) < 1e-3
+        assert abs(u.mean() - 0.5) < 1.5e-2
+        assert abs(u.std() - 1.0 / (2 * math.sqrt(3))) < 6e-3
+        states = cuda.random.create_xoroshiro128p_states(64, seed=1)
+        g = nrandom.xoroshiro128p_fill(states, out, 32, nrandom.NORMAL).copy_to_host()
+        assert abs(g.mean()) < 4e-3
+        assert abs(g.std() - 1.0) < 2e-3
+
+
+def test_float32_uniform_can_be_exactly_one_and_log_of_zero_is_unguarded():
+    # states chosen so that the first draw s0 + s1 is all ones / zero
+    st = np.zeros(2, nrandom.xoroshiro128p_dtype)
+    st[0] = (2**64 - 1, 0)       # draw = 2^64-1 -> 1.0f
+    st[1] = (0, 0)               # draw = 0      -> 0.0f -> log = -inf -> inf * cos
+    d = cuda.to_device(st)
+    out = cuda.device_array(2, np.float32)
+    nrandom.xoroshiro128p_fill(d, out, 1, nrandom.UNIFORM)
+    got = out.copy_to_host()
+    assert got[0] == np.float32(1.0) and got[1] == 0.0
+    d = cuda.to_device(st)
+    nrandom.xoroshiro128p_fill(d, out, 1, nrandom.NORMAL)
+    want, _ = cref.fill(st, 1, "normal_f32")
+    np.testing.assert_array_equal(out.copy_to_host(), want)
+
+
+def test_montecarlo_integration_end_to_end():
+    """docs example (tests/doc_examples/test_montecarlo.py:109-115): integral of
+    1/x over [1,2] and [2,3] with RNG + reduce, seed 42."""
+    n = 1_000_000
+    states = cuda.random.create_xoroshiro128p_states(n, seed=42)
+    u = cuda.device_array(n, np.float32)
+    nrandom.xoroshiro128p_fill(states, u, 1, nrandom.UNIFORM)
+    uh = u.copy_to_host().astype(np.float64)
+    for lo, hi, want in ((1, 2, 0.69315), (2, 3, 0.4055)):
+        y = (1.0 / (lo + uh * (hi - lo))).astype(np.float32)
+        est = cuda.reduce(lambda a, b: a + b)(cuda.to_device(y)) * (hi - lo) / n
+        assert abs(est - want) < 1e-3
+
+
+# ---- BASELINE config 4, full size -----------------------------------------------------
+
+@pytest.mark.parametrize("start", [0, 5])
+def test_config4_states_2_pow_24(start):
+    n = 2**24
+    states = cuda.random.create_xoroshiro128p_states(n, seed=42, subsequence_start=start)
+    got = states.copy_to_host()
+    _say("oracle chain for", n)
+    want = cref.init_states(n, 42, start)
+    assert got.tobytes() == want.tobytes()
+
+
+def test_config4_uniform_float32_2_pow_30_and_normal_float64():
+    n, count = 2**24, 64
+    host_states = cref.init_states(n, 42, 0)
+    states = cuda.to_device(host_states)
+    out = cuda.device_array(n * count, np.float32)
+    nrandom.xoroshiro128p_fill(states, out, count, nrandom.UNIFORM)
+    after = states.copy_to_host()
+    chunk = 2**20
+    for lo in range(0, n, chunk):
+        want, want_states = cref.fill(host_states[lo:lo + chunk], count, "uniform_f32")
+        got = out[lo * count:(lo + chunk) * count].copy_to_host()
+        assert got.tobytes() == want.tobytes(), lo
+        assert after[lo:lo + chunk].tobytes() == want_states.tobytes(), lo
+    del out
+    # separately, fresh states: 16 normal float64 per generator
+    states = cuda.to_device(host_states)
+    out = cuda.device_array(n * 16, np.float64)
+    nrandom.xoroshiro128p_fill(states, out, 16, nrandom.NORMAL)
+    after = states.copy_to_host()
+    worst = 0.0
+    for lo in range(0, n, chunk):
+        want, want_states = cref.fill(host_states[lo:lo + chunk], 16, "normal_f64")
+        got = out[lo * 16:(lo + chunk) * 16].copy_to_host()
+        worst = max(worst, _ulps(got, want).max())
+        assert after[lo:lo + chunk].tobytes() == want_states.tobytes(), lo
+    _say("normal_f64 worst ulp", worst)
+    assert worst <= 2.0

@@ -1,0 +1,176 @@
+"""Parity of Reduce (HIP path, through the C ABI) with the oracle.
+
+Bar: bit-exact for integers and for min/max; floating-point sums within
+|err| <= 2 n eps sum|x| of the exact sum AND of the value the reference's
+association order produces (oracle `tree`); products within 4 n eps relative.
+"""
+
+import math
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import numba_cuda_amd as cuda
+from oracle import cref
+
+sum_reduce = cuda.Reduce(lambda a, b: a + b)
+
+# numba_cuda/numba/cuda/tests/cudapy/test_reduction.py:29-45
+REFERENCE_SIZES = [1, 15, 16, 17, 127, 128, 129, 1023, 1024, 1025, 1536,
+                   1048576, 1049600, 1049728, 34567]
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.mark.parametrize("n", REFERENCE_SIZES)
+def test_sum_reduce_reference_sizes(n):
+    A = np.arange(n, dtype=np.float64) + 1
+    got = sum_reduce(A)
+    assert got == A.sum() == n * (n + 1) / 2
+    assert isinstance(got, np.float64)
+
+
+def test_empty_array_host_and_device():
+    A = np.arange(0, dtype=np.float64) + 1
+    assert sum_reduce(A) == 0
+    assert sum_reduce(cuda.to_device(A)) == 0
+    res = cuda.to_device(np.array([123.0]))
+    assert sum_reduce(A, res=res, init=7) == 7     # returns init, leaves res untouched
+    assert res[0] == 123.0
+
+
+def test_prod_max_min_init_res():
+    prod_reduce = cuda.reduce(lambda a, b: a * b)
+    A = np.arange(64, dtype=np.float64) + 1
+    np.testing.assert_allclose(prod_reduce(A, init=1), float(math.factorial(64)))
+    max_reduce = cuda.Reduce(lambda a, b: max(a, b))
+    B = np.arange(3717, dtype=np.float64) + 1
+    assert max_reduce(B, init=0) == 3717
+    assert cuda.Reduce(lambda a, b: min(a, b))(B, init=5000) == 1
+    C = np.arange(10, dtype=np.float64) + 1
+    assert sum_reduce(C, init=3) == C.sum() + 3
+    got = cuda.to_device(np.zeros(1, dtype=np.float64))
+    assert sum_reduce(C, res=got) is None
+    assert got[0] == C.sum()
+
+
+def test_only_1d_and_unknown_functor():
+    with pytest.raises(TypeError, match="only support 1D array"):
+        sum_reduce(np.zeros((2, 2)))
+    with pytest.raises(NotImplementedError):
+        cuda.Reduce(lambda a, b: a - b)
+
+
+def test_size_argument_and_offset_views():
+    rng = np.random.default_rng(1)
+    a = rng.integers(-1000, 1000, 5000).astype(np.int64)
+    d = cuda.to_device(a)
+    assert sum_reduce(d, size=1234) == a[:1234].sum()
+    assert sum_reduce(d, size=10**9) == a.sum()         # clamped like a slice
+    for lo in (1, 2, 3, 5, 127):
+        assert sum_reduce(d[lo:]) == a[lo:].sum()
+        assert sum_reduce(d[lo:4000 - lo]) == a[lo:4000 - lo].sum()
+    b = rng.integers(-100, 100, 3001).astype(np.int8)
+    db = cuda.to_device(b)
+    for lo in (0, 1, 7, 15, 16, 17):
+        assert sum_reduce(db[lo:]) == cref.fold("add", b[lo:])
+
+
+@pytest.mark.parametrize("sfx", list(cref.SUFFIX))
+@pytest.mark.parametrize("op", cref.OPS)
+def test_every_operator_and_dtype_against_oracle(op, sfx):
+    dt = np.dtype(cref.SUFFIX[sfx])
+    functor = {"add": lambda a, b: a + b, "mul": lambda a, b: a * b,
+               "max": lambda a, b: max(a, b), "min": lambda a, b: min(a, b)}[op]
+    red = cuda.Reduce(functor)
+    rng = np.random.default_rng(abs(hash((op, sfx))) % 2**32)
+    for n in (1, 7, 64, 65, 255, 256, 257, 4096, 65536, 300001, 2**21 + 3):
+        _say("reduce", op, sfx, n)
+        if dt.kind == "f":
+            a = rng.standard_normal(n).astype(dt) if op != "mul" else (1 + rng.standard_normal(n) * 1e-3).astype(dt)
+            init = 1.5
+        else:
+            info = np.iinfo(dt)
+            a = rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+            init = 3
+        got = red(a, init=init)
+        assert got.dtype == dt
+        if dt.kind == "f" and op == "add":
+            exact, sum_abs = cref.sum_exact(a)
+            tol = 2 * n * np.finfo(dt).eps * (sum_abs + 1.5)
+            assert abs(float(got) - (exact + 1.5)) <= tol
+            assert abs(float(got) - float(cref.tree(op, a, init))) <= 2 * tol
+        elif dt.kind == "f" and op == "mul":
+            assert abs(float(got) / float(cref.tree(op, a, init)) - 1) <= 4 * n * np.finfo(dt).eps
+        else:
+            assert got == cref.fold(op, a, init)
+            assert got == cref.tree(op, a, init)
+
+
+def test_runs_are_bitwise_reproducible():
+    rng = np.random.default_rng(5)
+    a = cuda.to_device(rng.standard_normal(3_000_017).astype(np.float32))
+    first = sum_reduce(a)
+    for _ in range(10):
+        assert sum_reduce(a).tobytes() == first.tobytes()
+
+
+def test_stream_and_result_slot_round_robin():
+    """BASELINE config 5 in small: independent row sums issued over 4 streams into
+    slots of one device vector."""
+    rng = np.random.default_rng(3)
+    rows, cols = 64, 65536
+    m = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
+    dm = cuda.to_device(m)
+    out = cuda.device_array(rows, dtype=np.float32)
+    streams = [cuda.stream() for _ in range(4)]
+    for i in range(rows):
+        assert sum_reduce(dm[i], res=out[i:i + 1], stream=streams[i % 4]) is None
+    for s in streams:
+        s.synchronize()
+    got = out.copy_to_host()
+    for i in range(rows):
+        exact, sum_abs = cref.sum_exact(m[i])
+        assert abs(float(got[i]) - exact) <= 2 * cols * np.finfo(np.float32).eps * sum_abs
+    # the same call returns the value when no `res` is given, also on a stream
+    v = sum_reduce(dm[5], stream=streams[1])
+    assert v.tobytes() == got[5].tobytes()
+
+
+# ---- BASELINE config 2: full HBM-scale inputs, seed 1 --------------------------------
+
+def test_config2_float32_sum_and_max_2_pow_28():
+    n = 2**28
+    _say("generating f32", n)
+    a = np.random.default_rng(1).standard_normal(n, dtype=np.float32)
+    d = cuda.to_device(a)
+    got = sum_reduce(d)
+    exact, sum_abs = cref.sum_exact(a)
+    tol = 2 * n * np.finfo(np.float32).eps * sum_abs
+    assert abs(float(got) - exact) <= tol
+    assert abs(float(got) - float(cref.tree("add", a))) <= 2 * tol
+    # in practice the tree order is far tighter than the bound; keep a tripwire
+    assert abs(float(got) - exact) <= 1e-3 * tol
+    mx = cuda.Reduce(lambda x, y: max(x, y))(d, init=-np.inf)
+    assert mx == a.max() == cref.tree("max", a, -np.inf)
+
+
+def test_config2_float64_sum_2_pow_27():
+    n = 2**27
+    a = np.random.default_rng(1).standard_normal(n)
+    got = sum_reduce(cuda.to_device(a))
+    exact, sum_abs = cref.sum_exact(a)
+    tol = 2 * n * np.finfo(np.float64).eps * sum_abs
+    assert abs(float(got) - exact) <= tol
+    assert abs(float(got) - float(cref.tree("add", a))) <= 2 * tol
+
+
+def test_config2_int64_sum_2_pow_28_bit_exact():
+    n = 2**28
+    a = np.random.default_rng(1).integers(-2**20, 2**20, n, dtype=np.int64, endpoint=True)
+    got = sum_reduce(cuda.to_device(a))
+    assert got == cref.tree("add", a) == a.sum()

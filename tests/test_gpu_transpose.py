@@ -1,0 +1,142 @@
+"""Parity of transpose (HIP path) with the oracle / numpy: bit-exact."""
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import numba_cuda_amd as cuda
+from numba_cuda_amd.kernels.transpose import transpose
+from oracle import cref
+
+recordwith2darray = np.dtype([("i", np.int32), ("j", np.float32, (3, 2))])
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _same_bytes(a, b):
+    return a.shape == b.shape and np.ascontiguousarray(a).tobytes() == np.ascontiguousarray(b).tobytes()
+
+
+@pytest.mark.parametrize("rows,cols,dtype", [(5, 6, np.float64), (128, 128, np.complex128),
+                                             (1025, 512, np.float64)])
+def test_transpose_reference_variants(rows, cols, dtype):
+    # numba_cuda/numba/cuda/tests/cudapy/test_transpose.py:17-32
+    x = np.arange(rows * cols, dtype=dtype).reshape(cols, rows)
+    y = np.zeros(rows * cols, dtype=dtype).reshape(rows, cols)
+    dx = cuda.to_device(x)
+    dy = cuda.cudadrv.devicearray.from_array_like(y)
+    assert transpose(dx, dy) is dy
+    dy.copy_to_host(y)
+    np.testing.assert_array_equal(x.transpose(), y)
+    np.testing.assert_array_equal(cref.transpose(x), y)
+
+
+SMALL = [(2, 3), (16, 16), (16, 17), (17, 16), (14, 15), (15, 14), (14, 14)]
+
+
+@pytest.mark.parametrize("rows,cols", SMALL)
+def test_transpose_record_and_bool(rows, cols):
+    arr = np.zeros((rows, cols), dtype=recordwith2darray)
+    for x in range(rows):
+        for y in range(cols):
+            arr[x, y]["i"] = x ** 2 + y
+            arr[x, y]["j"] = np.arange(6, dtype=np.float32).reshape(3, 2) * x + y
+    d_t = cuda.device_array_like(arr.T)
+    transpose(cuda.to_device(arr), d_t)
+    np.testing.assert_array_equal(arr.T, d_t.copy_to_host())
+    b = np.random.default_rng(rows * 31 + cols).integers(0, 2, (rows, cols)).astype(np.bool_)
+    d_b = cuda.device_array_like(b.T)
+    transpose(cuda.to_device(b), d_b)
+    np.testing.assert_array_equal(b.T, d_b.copy_to_host())
+
+
+def test_transpose_view():
+    # test_transpose.py:73-86
+    a = np.arange(120, dtype=np.int64).reshape((10, 12))
+    d_a = cuda.to_device(a)
+    d_t = d_a[::2, ::2].T
+    assert d_t.shape == (6, 5)
+    assert d_t.strides == (40, 8)
+    np.testing.assert_array_equal(a[::2, ::2].T, d_t.copy_to_host())
+    # negative and mixed strides, F order
+    np.testing.assert_array_equal(a[::-1, ::3].T, d_a[::-1, ::3].T.copy_to_host())
+    np.testing.assert_array_equal(a[1:, 2:].T, d_a[1:, 2:].T.copy_to_host())
+    f = np.asfortranarray(a)
+    np.testing.assert_array_equal(f.T, cuda.to_device(f).T.copy_to_host())
+
+
+def test_T_and_transpose_api():
+    a = np.arange(12, dtype=np.float32).reshape(3, 4)
+    d = cuda.to_device(a)
+    assert d.transpose((0, 1)) is d
+    with pytest.raises(ValueError, match="invalid axes list"):
+        d.transpose((0, 2))
+    with pytest.raises(NotImplementedError, match="non-2D"):
+        cuda.to_device(np.zeros(4)).T
+    np.testing.assert_array_equal(d.transpose((1, 0)).copy_to_host(), a.T)
+    # host arrays are accepted on both sides
+    out = np.zeros((4, 3), np.float32)
+    with pytest.warns(cuda.NumbaPerformanceWarning):
+        assert transpose(a, out) is out
+    np.testing.assert_array_equal(out, a.T)
+    with pytest.raises(ValueError, match="incompatible shape"):
+        transpose(d, cuda.device_array((3, 4), np.float32))
+    # empty
+    e = cuda.to_device(np.zeros((0, 5), np.float32)).T
+    assert e.shape == (5, 0)
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.uint16, np.float32, np.int64, np.complex128,
+                                   np.dtype("S3"), np.dtype("S12"), recordwith2darray])
+@pytest.mark.parametrize("shape", [(1, 1), (1, 300), (300, 1), (64, 64), (65, 63), (127, 129),
+                                   (257, 515), (1000, 777), (2049, 33)])
+def test_every_item_size_and_ragged_shapes(shape, dtype):
+    dtype = np.dtype(dtype)
+    _say("transpose", shape, dtype)
+    rng = np.random.default_rng(shape[0] * 7919 + shape[1])
+    a = rng.integers(0, 256, shape[0] * shape[1] * dtype.itemsize, dtype=np.uint8).view(dtype).reshape(shape)
+    got = cuda.to_device(a).T.copy_to_host()
+    assert _same_bytes(got, a.T)
+    assert _same_bytes(got, cref.transpose(a))
+
+
+def test_row_padded_inputs_and_outputs():
+    """Rows longer than the logical width on both sides (pitched allocations)."""
+    rng = np.random.default_rng(9)
+    big = rng.integers(0, 2**31, (300, 520), dtype=np.int32)
+    d_big = cuda.to_device(big)
+    src = d_big[:, 3:500]                       # row stride 520*4, misaligned start
+    dst_full = cuda.to_device(np.zeros((497, 333), np.int32))
+    dst = dst_full[:, 7:307]
+    transpose(src, dst)
+    want = np.zeros((497, 333), np.int32)
+    want[:, 7:307] = big[:, 3:500].T
+    np.testing.assert_array_equal(dst_full.copy_to_host(), want)
+
+
+# ---- BASELINE config 3, full size, seed 2 ------------------------------------------------
+
+def test_config3_float32_16384_square():
+    a = np.random.default_rng(2).random((16384, 16384), dtype=np.float32)
+    d = cuda.to_device(a)
+    t = d.T
+    got = t.copy_to_host()
+    assert _same_bytes(got, a.T)
+    back = t.T.copy_to_host()           # involution on the device
+    assert _same_bytes(back, a)
+
+
+def test_config3_float64_ragged_12345_by_6789():
+    a = np.random.default_rng(2).random((12345, 6789))
+    got = cuda.to_device(a).T.copy_to_host()
+    assert got.shape == (6789, 12345)
+    assert _same_bytes(got, a.T)
+
+
+def test_config3_int16_8192_by_32768():
+    a = np.random.default_rng(2).integers(-32768, 32767, (8192, 32768), dtype=np.int16, endpoint=True)
+    got = cuda.to_device(a).T.copy_to_host()
+    assert _same_bytes(got, a.T)
