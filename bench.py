@@ -1,0 +1,233 @@
+#!/usr/bin/env python
+"""Benchmark of the hot path on one MI355X.
+
+Default workload (BASELINE.json configs[1], the configuration the metric is quoted
+on): cuda.reduce float32 sum over 2^28 elements N(0,1), seed 1.  A "step" is one
+full reduction, issued through the public API into a device result slot; inputs
+are resident in HBM before the clock starts.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+Other workloads (--workload) report the same line for the remaining BASELINE
+configurations: reduce_f32_max, reduce_f64_sum, reduce_i64_sum, transpose_f32,
+transpose_f64, transpose_i16, rng_init, rng_uniform_f32, rng_normal_f64,
+batched_reduce.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E published peak
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (see profiles/); filled in per workload once measured, else None
+MEASURED_TRAFFIC = {}
+
+
+def _event_pair_times(cuda, stream, launch, reps):
+    """Average duration (ms) of one launch, from a HIP event pair around every
+    launch on the stream the kernel runs on."""
+    starts = [cuda.event(timing=True) for _ in range(reps)]
+    stops = [cuda.event(timing=True) for _ in range(reps)]
+    for i in range(reps):
+        starts[i].record(stream)
+        launch(i)
+        stops[i].record(stream)
+    stream.synchronize()
+    times = [starts[i].elapsed_time(stops[i]) for i in range(reps)]
+    return float(np.mean(times)), float(np.min(times)), float(np.median(times))
+
+
+def _cpu_baseline_reduce(a_host, target_seconds=12.0):
+    """The reference's CPU path for reduce (its simulator: a left fold through the
+    Python functor, one call per element, single core by construction), timed on a
+    bounded prefix of the same input."""
+    from oracle import sim
+    red = sim.Reduce(lambda x, y: x + y)
+    probe = a_host[:1 << 18]
+    t0 = time.perf_counter()
+    red(probe, init=0)
+    per_elem = (time.perf_counter() - t0) / probe.size
+    n = int(min(a_host.size, max(1 << 18, target_seconds / per_elem)))
+    n = 1 << (n.bit_length() - 1)
+    sample = a_host[:n]
+    t0 = time.perf_counter()
+    red(sample, init=0)
+    dt = time.perf_counter() - t0
+    return {"value": round(sample.nbytes / dt / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "first 2^%d float32 elements of the same input, simulator-style left fold "
+                      "(functools.reduce over NumPy scalars), %.1f s" % (n.bit_length() - 1, dt),
+            "elements_per_s": round(n / dt, 1), "host_cores_available": os.cpu_count()}
+
+
+def _workload(name, cuda):
+    """-> dict(desc, dtype, algo_bytes, units, step(i), stream, host_input, kernel)"""
+    from numba_cuda_amd import random as nrandom
+    from numba_cuda_amd.kernels.transpose import transpose
+    stream = cuda.stream()
+    add = cuda.Reduce(lambda a, b: a + b)
+    mx = cuda.Reduce(lambda a, b: max(a, b))
+    rng = np.random.default_rng(1)
+    if name.startswith("reduce_"):
+        if name == "reduce_f32_sum" or name == "reduce_f32_max":
+            host = rng.standard_normal(2**28, dtype=np.float32)
+            desc = "cuda.reduce fp32 %s, 2^28 elements N(0,1), seed 1" % ("sum" if name.endswith("sum") else "max")
+        elif name == "reduce_f64_sum":
+            host = rng.standard_normal(2**27)
+            desc = "cuda.reduce fp64 sum, 2^27 elements N(0,1), seed 1"
+        elif name == "reduce_i64_sum":
+            host = rng.integers(-2**20, 2**20, 2**28, dtype=np.int64, endpoint=True)
+            desc = "cuda.reduce int64 sum, 2^28 elements in [-2^20, 2^20], seed 1"
+        else:
+            raise SystemExit("unknown workload %s" % name)
+        # two resident copies, alternated, so no launch can be served from the
+        # 256 MB Infinity Cache by its predecessor
+        bufs = [cuda.to_device(host), cuda.to_device(host)]
+        res = cuda.device_array(1, dtype=host.dtype)
+        red = mx if name.endswith("max") else add
+        init = -np.inf if name.endswith("max") else 0
+
+        def step(i):
+            red(bufs[i & 1], res=res, init=init, stream=stream)
+
+        return dict(desc=desc, dtype={"float32": "f32", "float64": "f64", "int64": "int64"}[host.dtype.name],
+                    algo_bytes=host.nbytes, units=host.size, step=step, stream=stream, host=host,
+                    kernel="reduce_kernel", keep=(bufs, res))
+    if name.startswith("transpose_"):
+        rng = np.random.default_rng(2)
+        if name == "transpose_f32":
+            host = rng.random((16384, 16384), dtype=np.float32)
+        elif name == "transpose_f64":
+            host = rng.random((12345, 6789))
+        elif name == "transpose_i16":
+            host = rng.integers(-32768, 32767, (8192, 32768), dtype=np.int16, endpoint=True)
+        else:
+            raise SystemExit("unknown workload %s" % name)
+        src = cuda.to_device(host).bind(stream)
+        dst = cuda.device_array((host.shape[1], host.shape[0]), dtype=host.dtype, stream=stream)
+
+        def step(i):
+            transpose(src, dst)
+
+        return dict(desc="transpose %s %dx%d, seed 2" % (host.dtype.name, host.shape[0], host.shape[1]),
+                    dtype=host.dtype.name, algo_bytes=2 * host.nbytes, units=host.size, step=step,
+                    stream=stream, host=None, kernel="transpose_tiled", keep=(src, dst))
+    if name.startswith("rng_"):
+        n = 2**24
+        states = cuda.device_array(n, dtype=nrandom.xoroshiro128p_dtype)
+        nrandom.init_xoroshiro128p_states(states, 42)
+        if name == "rng_init":
+            def step(i):
+                nrandom.init_xoroshiro128p_states(states, 42, 0, stream)
+            return dict(desc="create_xoroshiro128p_states 2^24 states, seed 42", dtype="u64",
+                        algo_bytes=16 * n, units=n, step=step, stream=stream, host=None,
+                        kernel="init_states_kernel", keep=(states,))
+        if name == "rng_uniform_f32":
+            out = cuda.device_array(n * 64, np.float32)
+
+            def step(i):
+                nrandom.xoroshiro128p_fill(states, out, 64, nrandom.UNIFORM, stream)
+            return dict(desc="xoroshiro128p 2^24 generators x 64 uniform float32", dtype="u64",
+                        algo_bytes=4 * n * 64 + 32 * n, units=n * 64, step=step, stream=stream, host=None,
+                        kernel="fill_kernel", keep=(states, out))
+        if name == "rng_normal_f64":
+            out = cuda.device_array(n * 16, np.float64)
+
+            def step(i):
+                nrandom.xoroshiro128p_fill(states, out, 16, nrandom.NORMAL, stream)
+            return dict(desc="xoroshiro128p 2^24 generators x 16 normal float64", dtype="f64",
+                        algo_bytes=8 * n * 16 + 32 * n, units=n * 16, step=step, stream=stream, host=None,
+                        kernel="fill_kernel", keep=(states, out))
+    if name == "batched_reduce":
+        rows, cols = 4096, 65536
+        host = np.random.default_rng(3).uniform(-1, 1, (rows, cols)).astype(np.float32)
+        dm = cuda.to_device(host)
+        out = cuda.device_array(rows, np.float32)
+        streams = [cuda.stream() for _ in range(4)]
+        views = [dm[i] for i in range(rows)]
+        slots = [out[i:i + 1] for i in range(rows)]
+
+        def step(i):
+            for r in range(rows):
+                add(views[r], res=slots[r], stream=streams[r & 3])
+            for s in streams[1:]:
+                s.synchronize()
+
+        return dict(desc="4096 x (65536 fp32) row sums round-robin over 4 streams, seed 3", dtype="f32",
+                    algo_bytes=host.nbytes, units=rows, step=step, stream=streams[0], host=None,
+                    kernel="reduce_kernel", keep=(dm, out, streams, views, slots), calls_per_step=rows)
+    raise SystemExit("unknown workload %s" % name)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="reduce_f32_sum")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
+                         "(run with --gpus 1)")
+
+    import numba_cuda_amd as cuda
+    if not cuda.is_available():
+        raise SystemExit("no GPU / HIP library: %s" % cuda.cuda_error())
+    w = _workload(args.workload, cuda)
+    stream, step = w["stream"], w["step"]
+
+    for i in range(args.warmup):
+        step(i)
+    stream.synchronize()
+    cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    stream.synchronize()
+    cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    gbs = w["algo_bytes"] / (ms_per_step * 1e-3) / 1e9
+
+    roofline = None
+    if "calls_per_step" not in w:
+        mean_ms, min_ms, med_ms = _event_pair_times(cuda, stream, step, min(args.steps, 200))
+        achieved = w["algo_bytes"] / (mean_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
+                    "kernel": w["kernel"], "algorithmic_bytes_per_launch": w["algo_bytes"],
+                    "launch_ms_mean": round(mean_ms, 5), "launch_ms_min": round(min_ms, 5),
+                    "launch_ms_median": round(med_ms, 5)}
+
+    cpu = None
+    if args.workload == "reduce_f32_sum" and not args.no_cpu_baseline:
+        cpu = _cpu_baseline_reduce(w["host"])
+
+    line = {
+        "metric": "achieved HBM GB/s (% of 8 TB/s) for cuda.reduce fp32 sum at 2^28 elems"
+        if args.workload == "reduce_f32_sum" else "achieved HBM GB/s for " + args.workload,
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": w["desc"], "name": args.workload},
+        "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "units_per_s": round(w["units"] / (ms_per_step * 1e-3), 1),
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+    if "calls_per_step" in w:
+        line["us_per_call"] = round(ms_per_step * 1e3 / w["calls_per_step"], 3)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

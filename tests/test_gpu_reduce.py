@@ -174,3 +174,28 @@ def test_config2_int64_sum_2_pow_28_bit_exact():
     a = np.random.default_rng(1).integers(-2**20, 2**20, n, dtype=np.int64, endpoint=True)
     got = sum_reduce(cuda.to_device(a))
     assert got == cref.tree("add", a) == a.sum()
+
+
+def test_back_to_back_reductions_never_see_stale_partials():
+    """Thousands of launches reuse one scratch buffer per stream with different
+    data each time; a partial read from a stale cache line would change an integer
+    sum.  Sizes span 2 to 512 workgroups."""
+    rng = np.random.default_rng(77)
+    n_max = 3_000_000
+    base = rng.integers(-2**40, 2**40, n_max + 4096, dtype=np.int64)
+    d = cuda.to_device(base)
+    calls = 3000
+    offs = rng.integers(0, 4096, calls)
+    sizes = rng.integers(5000, n_max, calls)
+    sizes[::7] = rng.integers(2_500_000, n_max, len(sizes[::7]))
+    out = cuda.device_array(calls, np.int64)
+    streams = [cuda.stream() for _ in range(3)]
+    for i in range(calls):
+        sum_reduce(d[offs[i]:offs[i] + sizes[i]], res=out[i:i + 1], init=i, stream=streams[i % 3])
+    for s in streams:
+        s.synchronize()
+    got = out.copy_to_host()
+    csum = np.concatenate([[0], np.cumsum(base)])
+    want = csum[offs + sizes] - csum[offs] + np.arange(calls)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, (bad[:10], got[bad[:10]], want[bad[:10]])
