@@ -33,18 +33,18 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E published peak
 MEASURED_TRAFFIC = {}
 
 
-def _event_pair_times(cuda, stream, launch, reps):
-    """Average duration (ms) of one launch, from a HIP event pair around every
-    launch on the stream the kernel runs on."""
-    starts = [cuda.event(timing=True) for _ in range(reps)]
-    stops = [cuda.event(timing=True) for _ in range(reps)]
+def _event_timed_launches(cuda, stream, launch, reps):
+    """Average duration (ms) of one launch: one HIP event pair, recorded on the
+    stream the kernels run on, around `reps` back-to-back launches.  Launches on one
+    stream run one after another, so elapsed / reps is the per-launch duration
+    including the (sub-microsecond) hand-over between consecutive kernels."""
+    start, stop = cuda.event(timing=True), cuda.event(timing=True)
+    start.record(stream)
     for i in range(reps):
-        starts[i].record(stream)
         launch(i)
-        stops[i].record(stream)
-    stream.synchronize()
-    times = [starts[i].elapsed_time(stops[i]) for i in range(reps)]
-    return float(np.mean(times)), float(np.min(times)), float(np.median(times))
+    stop.record(stream)
+    stop.synchronize()
+    return start.elapsed_time(stop) / reps
 
 
 def _cpu_baseline_reduce(a_host, target_seconds=12.0):
@@ -201,13 +201,12 @@ def main():
 
     roofline = None
     if "calls_per_step" not in w:
-        mean_ms, min_ms, med_ms = _event_pair_times(cuda, stream, step, min(args.steps, 200))
-        achieved = w["algo_bytes"] / (mean_ms * 1e-3) / 1e9
+        launch_ms = _event_timed_launches(cuda, stream, step, args.steps)
+        achieved = w["algo_bytes"] / (launch_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
                     "kernel": w["kernel"], "algorithmic_bytes_per_launch": w["algo_bytes"],
-                    "launch_ms_mean": round(mean_ms, 5), "launch_ms_min": round(min_ms, 5),
-                    "launch_ms_median": round(med_ms, 5)}
+                    "launch_us_avg": round(launch_ms * 1e3, 2), "launches_timed": args.steps}
 
     cpu = None
     if args.workload == "reduce_f32_sum" and not args.no_cpu_baseline:

@@ -101,7 +101,6 @@ def _merge_groups(old_shape, old_strides, new_shape, itemsize, fortran):
                     return None
             elif a[1] != b[0] * b[1]:
                 return None
-        dims = new_shape[ni:nj]
         if fortran:
             acc = run[0][1]
             for k in range(ni, nj):
@@ -112,7 +111,6 @@ def _merge_groups(old_shape, old_strides, new_shape, itemsize, fortran):
             for k in range(nj - 1, ni - 1, -1):
                 new_strides[k] = acc
                 acc *= new_shape[k]
-        del dims
         oi, ni = oj, nj
     # whatever is left of the new shape is length-1 axes
     if ni >= 1:
@@ -261,8 +259,10 @@ class Array:
             raise ValueError("reshape changes the size of the array")
         if order == "A":
             order = "F" if self.is_f_contig else "C"
-        if self.is_c_contig or self.is_f_contig:
-            newstrides = (c_strides if order == "C" else f_strides)(newdims, self.itemsize)
+        if order == "C" and self.is_c_contig:
+            newstrides = c_strides(newdims, self.itemsize)
+        elif order == "F" and self.is_f_contig:
+            newstrides = f_strides(newdims, self.itemsize)
         elif self.size == 0:
             newstrides = (self.itemsize,) * len(newdims)
         else:

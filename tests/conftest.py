@@ -23,3 +23,36 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def fake_gpu(monkeypatch):
+    """The driver layer bound to tests/fakelib.FakeLib: device memory lives in
+    host RAM, no kernels exist.  Yields the FakeLib for inspection."""
+    from tests.fakelib import FakeLib
+    from numba_cuda_amd.cudadrv import devices, driver as drv
+
+    lib = FakeLib()
+    d = drv.driver
+    saved = dict(d.__dict__)
+    for name in [k for k in d.__dict__ if k.startswith("nbh_")]:
+        del d.__dict__[name]                      # drop cached checked wrappers
+    d.lib, d.is_initialized, d.initialization_error, d.pid = lib, True, None, os.getpid()
+    d.get_device.cache_clear()
+    devices._runtime._tls.__dict__.clear()
+    if "lst" in devices.gpus.__dict__:
+        del devices.gpus.__dict__["lst"]
+    monkeypatch.setattr(drv, "_memory_manager", None)
+    try:
+        yield lib
+    finally:
+        import gc
+        gc.collect()
+        d.__dict__.clear()
+        d.__dict__.update(saved)
+        for name in [k for k in d.__dict__ if k.startswith("nbh_")]:
+            del d.__dict__[name]
+        d.get_device.cache_clear()
+        devices._runtime._tls.__dict__.clear()
+        if "lst" in devices.gpus.__dict__:
+            del devices.gpus.__dict__["lst"]
