@@ -144,6 +144,19 @@ int nbh_transpose(const void *in, void *out, int64_t rows, int64_t cols, int64_t
                   int64_t in_stride1, int64_t out_stride0, int64_t out_stride1, int64_t itemsize,
                   nbh_stream_t stream);
 
+/* ---- strided assignment ---------------------------------------------------- */
+
+#define NBH_ASSIGN_MAX_NDIM 8
+
+/* cudadrv/devicearray.py:534-575 _assign_kernel and :741-790 _do_setitem (the
+ * device side of `darr[key] = value`): dst[i0..ik] = src[i0..ik] for every index
+ * of `shape` (ndim <= NBH_ASSIGN_MAX_NDIM), items of `itemsize` bytes, byte
+ * strides arbitrary on both sides; a source stride of 0 broadcasts that axis.
+ * Contiguous-to-contiguous assignments run as a flat 128-bit copy.  Source and
+ * destination must not overlap. */
+int nbh_assign(void *dst, const void *src, int ndim, const int64_t *shape, const int64_t *dst_strides,
+               const int64_t *src_strides, int64_t itemsize, nbh_stream_t stream);
+
 /* ---- xoroshiro128+ -------------------------------------------------------- */
 
 /* random.py:241-282 init_xoroshiro128p_states (the sequential CPU jump chain plus

@@ -1,0 +1,168 @@
+// nbh_assign: dst[i0, ..., ik] = src[i0, ..., ik] over an n-d index space, with
+// arbitrary byte strides on both sides (a zero source stride broadcasts).
+//
+// The host first squeezes the index space: axes of length 1 vanish and neighbouring
+// axes that are laid out back to back on both sides fuse.  What is left decides
+// the kernel:
+//   * one axis with unit stride on both sides -> a flat copy: 16-byte packets,
+//     grid-stride, the ragged tail done item by item
+//   * anything else -> one lane per chunk of an item, innermost axis fastest
+//
+// HBM roofline of the flat copy: bytes read + bytes written = 2 * n * itemsize.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxDims = NBH_ASSIGN_MAX_NDIM;
+
+struct alignas(16) Chunk16 {
+    uint32_t w[4];
+};
+template <int G> struct ChunkOf;
+template <> struct ChunkOf<1> { using type = uint8_t; };
+template <> struct ChunkOf<2> { using type = uint16_t; };
+template <> struct ChunkOf<4> { using type = uint32_t; };
+template <> struct ChunkOf<8> { using type = uint64_t; };
+template <> struct ChunkOf<16> { using type = Chunk16; };
+
+// 16 bytes that are only aligned to G
+template <int G> struct __attribute__((packed, aligned(G))) Packet {
+    typename ChunkOf<G>::type c[16 / G];
+};
+
+template <int G>
+__global__ __launch_bounds__(kThreads) void copy_flat(char *__restrict__ dst, const char *__restrict__ src,
+                                                      int64_t nbytes)
+{
+    const int64_t npack = nbytes / 16;
+    const int64_t step = (int64_t)gridDim.x * kThreads;
+    const int64_t first = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    for (int64_t i = first; i < npack; i += step)
+        *reinterpret_cast<Packet<G> *>(dst + i * 16) = *reinterpret_cast<const Packet<G> *>(src + i * 16);
+    using C = typename ChunkOf<G>::type;
+    for (int64_t b = npack * 16 + first * G; b < nbytes; b += step * G)
+        *reinterpret_cast<C *>(dst + b) = *reinterpret_cast<const C *>(src + b);
+}
+
+struct Dims {
+    int nd;
+    int64_t shape[kMaxDims];
+    int64_t dst_stride[kMaxDims];
+    int64_t src_stride[kMaxDims];
+};
+
+template <int G>
+__global__ __launch_bounds__(kThreads) void copy_strided(char *__restrict__ dst, const char *__restrict__ src,
+                                                         Dims d, int64_t chunks, int64_t total)
+{
+    using C = typename ChunkOf<G>::type;
+    const int64_t step = (int64_t)gridDim.x * kThreads;
+    for (int64_t id = (int64_t)blockIdx.x * kThreads + threadIdx.x; id < total; id += step) {
+        int64_t rest = id / chunks;
+        int64_t doff = (id % chunks) * G, soff = doff;
+        for (int k = d.nd - 1; k >= 0; --k) {
+            const int64_t i = rest % d.shape[k];
+            rest /= d.shape[k];
+            doff += i * d.dst_stride[k];
+            soff += i * d.src_stride[k];
+        }
+        *reinterpret_cast<C *>(dst + doff) = *reinterpret_cast<const C *>(src + soff);
+    }
+}
+
+inline int64_t low_bit(uint64_t x) { return (int64_t)(x & (~x + 1)); }
+
+template <int G> int launch_flat(void *dst, const void *src, int64_t nbytes, hipStream_t s)
+{
+    int64_t grid = (nbytes / 16 + kThreads - 1) / kThreads;
+    const int64_t cap = (int64_t)nbh_cu_count() * 8;
+    if (grid > cap)
+        grid = cap;
+    if (grid < 1)
+        grid = 1;
+    hipLaunchKernelGGL((copy_flat<G>), dim3((unsigned)grid), dim3(kThreads), 0, s, (char *)dst, (const char *)src,
+                       nbytes);
+    return nbh_launch_status();
+}
+
+template <int G>
+int launch_strided(void *dst, const void *src, const Dims &d, int64_t itemsize, int64_t items, hipStream_t s)
+{
+    const int64_t chunks = itemsize / G;
+    const int64_t total = items * chunks;
+    int64_t grid = (total + kThreads - 1) / kThreads;
+    const int64_t cap = (int64_t)nbh_cu_count() * 32;
+    if (grid > cap)
+        grid = cap;
+    hipLaunchKernelGGL((copy_strided<G>), dim3((unsigned)grid), dim3(kThreads), 0, s, (char *)dst,
+                       (const char *)src, d, chunks, total);
+    return nbh_launch_status();
+}
+
+}  // namespace
+
+extern "C" int nbh_assign(void *dst, const void *src, int ndim, const int64_t *shape, const int64_t *dst_strides,
+                          const int64_t *src_strides, int64_t itemsize, nbh_stream_t stream)
+{
+    if (ndim < 0 || ndim > kMaxDims || itemsize < 1 || (ndim > 0 && (!shape || !dst_strides || !src_strides)))
+        return (int)hipErrorInvalidValue;
+    int64_t items = 1;
+    for (int k = 0; k < ndim; ++k) {
+        if (shape[k] < 0)
+            return (int)hipErrorInvalidValue;
+        items *= shape[k];
+    }
+    if (items == 0)
+        return 0;
+    if (!dst || !src)
+        return (int)hipErrorInvalidValue;
+
+    // squeeze: drop unit axes, fuse axes that continue each other on both sides
+    Dims d;
+    d.nd = 0;
+    for (int k = 0; k < ndim; ++k) {
+        if (shape[k] == 1)
+            continue;
+        if (d.nd > 0 && d.dst_stride[d.nd - 1] == dst_strides[k] * shape[k] &&
+            d.src_stride[d.nd - 1] == src_strides[k] * shape[k]) {
+            d.shape[d.nd - 1] *= shape[k];
+            d.dst_stride[d.nd - 1] = dst_strides[k];
+            d.src_stride[d.nd - 1] = src_strides[k];
+        } else {
+            d.shape[d.nd] = shape[k];
+            d.dst_stride[d.nd] = dst_strides[k];
+            d.src_stride[d.nd] = src_strides[k];
+            ++d.nd;
+        }
+    }
+    for (int k = d.nd; k < kMaxDims; ++k) {
+        d.shape[k] = 1;
+        d.dst_stride[k] = d.src_stride[k] = 0;
+    }
+
+    uint64_t mix = (uint64_t)itemsize | (uint64_t)(uintptr_t)dst | (uint64_t)(uintptr_t)src | 16u;
+    for (int k = 0; k < d.nd; ++k)
+        mix |= (uint64_t)d.dst_stride[k] | (uint64_t)d.src_stride[k];
+    const int64_t g = low_bit(mix);
+    hipStream_t s = nbh_hip_stream(stream);
+
+    const bool flat = d.nd == 0 || (d.nd == 1 && d.dst_stride[0] == itemsize && d.src_stride[0] == itemsize);
+    if (flat) {
+        const int64_t nbytes = items * itemsize;
+        switch (g) {
+        case 1: return launch_flat<1>(dst, src, nbytes, s);
+        case 2: return launch_flat<2>(dst, src, nbytes, s);
+        case 4: return launch_flat<4>(dst, src, nbytes, s);
+        case 8: return launch_flat<8>(dst, src, nbytes, s);
+        default: return launch_flat<16>(dst, src, nbytes, s);
+        }
+    }
+    switch (g) {
+    case 1: return launch_strided<1>(dst, src, d, itemsize, items, s);
+    case 2: return launch_strided<2>(dst, src, d, itemsize, items, s);
+    case 4: return launch_strided<4>(dst, src, d, itemsize, items, s);
+    case 8: return launch_strided<8>(dst, src, d, itemsize, items, s);
+    default: return launch_strided<16>(dst, src, d, itemsize, items, s);
+    }
+}

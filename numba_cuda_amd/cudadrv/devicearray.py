@@ -9,6 +9,7 @@ memory if it has a truthy `__cuda_memory__`; it is a device array if it also has
 """
 
 import copy
+import ctypes
 import functools
 import math
 from ctypes import c_void_p
@@ -362,8 +363,52 @@ class DeviceNDArray(DeviceNDArrayBase):
         return self._do_setitem(key, value, stream=stream)
 
     def _do_setitem(self, key, value, stream=0):
-        raise NotImplementedError("item assignment on device arrays is not part of this build; "
-                                  "copy with copy_to_device() instead")
+        stream = self._default_stream(stream)
+        # no stream bound and none given: work on the default stream and wait for it
+        synchronous = not stream
+        if synchronous:
+            stream = devices.get_context().get_default_stream()
+
+        # left-hand side: a view of the selected items (0-d for a single item)
+        arr = self._dummy.__getitem__(key)
+        newdata = self.gpu_data.view(*arr.extent)
+        if isinstance(arr, dummyarray.Element):
+            shape, strides = (), ()
+        else:
+            shape, strides = arr.shape, arr.strides
+        lhs = type(self)(shape=shape, strides=strides, dtype=self.dtype, gpu_data=newdata, stream=stream)
+
+        # right-hand side: on the device, padded with leading unit axes, broadcastable
+        if not _driver.is_device_memory(value) and not hasattr(value, "__cuda_array_interface__"):
+            # host values take the dtype of the target, as a NumPy assignment would
+            value = np.asarray(value).astype(self.dtype, copy=False)
+        rhs, _ = auto_device(value, stream=stream, user_explicit=True)
+        if rhs.ndim > lhs.ndim:
+            raise ValueError("Can't assign %s-D array to %s-D self" % (rhs.ndim, lhs.ndim))
+        if rhs.dtype != lhs.dtype:
+            raise TypeError("incompatible dtype: %s vs. %s" % (lhs.dtype, rhs.dtype))
+        pad = lhs.ndim - rhs.ndim
+        rhs_shape = (1,) * pad + tuple(rhs.shape)
+        rhs_strides = (0,) * pad + tuple(rhs.strides)
+        for i, (l, r) in enumerate(zip(lhs.shape, rhs_shape)):
+            if r != 1 and l != r:
+                raise ValueError("Can't copy sequence with size %d to array "
+                                 "axis %d with dimension %d" % (r, i, l))
+        # a unit axis on the right repeats along the matching axis on the left
+        src_strides = tuple(0 if r == 1 else s for r, s in zip(rhs_shape, rhs_strides))
+
+        nd = lhs.ndim
+        if nd > _MAX_ASSIGN_NDIM:
+            raise NotImplementedError("assignment supports at most %d axes" % _MAX_ASSIGN_NDIM)
+        vec = ctypes.c_int64 * max(nd, 1)
+        _driver.driver.nbh_assign(lhs.device_ctypes_pointer.value, rhs.device_ctypes_pointer.value, nd,
+                                  vec(*lhs.shape), vec(*lhs.strides), vec(*src_strides),
+                                  self.dtype.itemsize, _driver._stream_handle(stream) or None)
+        if synchronous:
+            stream.synchronize()
+
+
+_MAX_ASSIGN_NDIM = 8
 
 
 class MappedNDArray(DeviceNDArrayBase, np.ndarray):

@@ -16,6 +16,17 @@ def _gpu_present():
     return os.path.exists("/dev/kfd")
 
 
+if _gpu_present():
+    # PyTorch-ROCm wheels bundle their own HIP runtime under an unversioned file
+    # name.  Loaded first, it is shared by libnbhip.so (same SONAME); loaded second,
+    # the process ends up with two HIP runtimes and torch no longer sees the GPU.
+    # The interop test needs both, so torch goes first.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+
+
 def pytest_collection_modifyitems(config, items):
     if _gpu_present():
         return

@@ -50,3 +50,55 @@ def test_cuda_array_interface_with_torch_tensors():
     assert torch.equal(back, t.t().contiguous())
     with pytest.raises(TypeError):
         cuda.as_cuda_array(np.zeros(3))
+
+
+def test_setitem_scalars_rows_columns_broadcast():
+    """`darr[key] = value` (reference: tests/cudadrv/test_cuda_array_slicing.py:220-379)."""
+    a = np.arange(5 * 7, dtype=np.float64).reshape(5, 7)
+    d = cuda.to_device(a)
+    d[2, 3] = 500
+    a[2, 3] = 500
+    d[1] = np.arange(7) * 10.0
+    a[1] = np.arange(7) * 10.0
+    d[:, 2] = 3.5                                   # scalar broadcast over a strided column
+    a[:, 2] = 3.5
+    d[:, 4] = np.arange(5.0)                        # 1-d into a column
+    a[:, 4] = np.arange(5.0)
+    d[3:, 5:] = cuda.to_device(np.full((2, 2), -1.0))   # device source
+    a[3:, 5:] = -1.0
+    d[::2, ::3] = np.array([[9.0], [8.0], [7.0]])   # broadcast along the inner axis
+    a[::2, ::3] = np.array([[9.0], [8.0], [7.0]])
+    d[4] = 7                                        # int value into a float array
+    a[4] = 7
+    np.testing.assert_array_equal(d.copy_to_host(), a)
+    d[:] = 0.25
+    assert (d.copy_to_host() == 0.25).all()
+    with pytest.raises(ValueError, match="Can't assign 3-D array to 2-D self"):
+        d[:] = np.zeros((1, 5, 7))
+    with pytest.raises(ValueError, match="Can't copy sequence with size 3 to array axis 1 with dimension 7"):
+        d[:] = np.zeros((5, 3))
+    with pytest.raises(IndexError):
+        d[5, 0] = 1.0
+    # on a stream: asynchronous, same result
+    s = cuda.stream()
+    d.setitem((slice(None), 0), np.arange(5.0) + 100, stream=s)
+    s.synchronize()
+    np.testing.assert_array_equal(d.copy_to_host()[:, 0], np.arange(5.0) + 100)
+    # other item sizes, many axes, big flat copy
+    for dt in (np.int8, np.int16, np.complex128, np.dtype([("i", np.int32), ("j", np.float32, (3, 2))])):
+        rng = np.random.default_rng(0)
+        dt = np.dtype(dt)
+        h = rng.integers(0, 255, 4 * 3 * 5 * 6 * dt.itemsize, dtype=np.uint8).view(dt).reshape(4, 3, 5, 6)
+        z = cuda.to_device(np.zeros_like(h))
+        z[1:, :, ::2, 1:5] = np.ascontiguousarray(h[1:, :, ::2, 1:5])   # host sources must be contiguous
+        with pytest.raises(ValueError, match="non-contiguous buffer"):
+            z[1:, :, ::2, 1:5] = h[1:, :, ::2, 1:5]
+        want = np.zeros_like(h)
+        want[1:, :, ::2, 1:5] = h[1:, :, ::2, 1:5]
+        assert z.copy_to_host().tobytes() == want.tobytes()
+    big = np.random.default_rng(1).integers(0, 2**31, 3_000_001, dtype=np.int32)
+    t = cuda.device_array_like(big)
+    t[:] = cuda.to_device(big)
+    np.testing.assert_array_equal(t.copy_to_host(), big)
+    t[1:] = cuda.to_device(big)[:-1]                 # misaligned flat copy
+    np.testing.assert_array_equal(t.copy_to_host()[1:], big[:-1])
