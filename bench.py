@@ -11,7 +11,7 @@ are resident in HBM before the clock starts.  Prints ONE JSON line.
 Other workloads (--workload) report the same line for the remaining BASELINE
 configurations: reduce_f32_max, reduce_f64_sum, reduce_i64_sum, transpose_f32,
 transpose_f64, transpose_i16, rng_init, rng_uniform_f32, rng_normal_f64,
-batched_reduce.
+batched_reduce, copy_f32 (counter calibration).
 """
 
 import argparse
@@ -30,7 +30,12 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E published peak
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (see profiles/); filled in per workload once measured, else None
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 779 029 B fetched + 32 832 B written
+    "reduce_f32_sum": 1073811861,
+    # profiles/copy_flat_f32_2p28.txt: the calibration kernel itself
+    "copy_f32": 2147483648,
+}
 
 
 def _event_timed_launches(cuda, stream, launch, reps):
@@ -147,6 +152,20 @@ def _workload(name, cuda):
             return dict(desc="xoroshiro128p 2^24 generators x 16 normal float64", dtype="f64",
                         algo_bytes=8 * n * 16 + 32 * n, units=n * 16, step=step, stream=stream, host=None,
                         kernel="fill_kernel", keep=(states, out))
+    if name == "copy_f32":
+        # flat device-to-device assignment: the plain copy kernel of known size that
+        # the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are calibrated against
+        host = np.random.default_rng(4).random(2**28, dtype=np.float32)
+        src = cuda.to_device(host)
+        dst = cuda.device_array_like(host)
+        everything = slice(None)
+
+        def step(i):
+            dst.setitem(everything, src, stream=stream)
+
+        return dict(desc="flat copy dst[:] = src, 2^28 float32 (counter calibration)", dtype="u8",
+                    algo_bytes=2 * host.nbytes, units=host.size, step=step, stream=stream, host=None,
+                    kernel="copy_flat", keep=(src, dst))
     if name == "batched_reduce":
         rows, cols = 4096, 65536
         host = np.random.default_rng(3).uniform(-1, 1, (rows, cols)).astype(np.float32)
