@@ -1,17 +1,29 @@
 // nbh_transpose: out[j, i] = in[i, j] for items of any size and any byte strides.
 //
 // Two kernels:
-//   * tiled  - item size 1, 2, 4, 8 or 16 bytes with unit inner stride on both
-//              sides (row strides free).  A workgroup moves one tile whose rows
-//              are 256 bytes long on the input side and on the output side: it
-//              reads the tile with 128-bit loads along input rows, parks it in
-//              LDS (row pitch padded by one item against bank conflicts), and
-//              writes it with 128-bit stores along output rows.  Ragged edge
-//              tiles fall back to per-item accesses only for the vectors that
-//              stick out.
+//   * packets - item size 1, 2, 4, 8 or 16 bytes with unit inner stride on both
+//               sides (row strides free).  Every lane moves V x V items, V = 16 /
+//               itemsize: it loads one 16-byte packet from each of V consecutive
+//               input rows, transposes the V x V block in registers, and stores one
+//               packet to each of V consecutive output rows.  The 64 lanes of a
+//               wavefront form an 8 x 8 grid, so each load and each store
+//               instruction covers eight whole 128-byte lines: no LDS, no barrier.
+//               A workgroup covers a tall tile (many input rows, few columns) and
+//               consecutive workgroups walk DOWN the input, i.e. ALONG the output
+//               rows: what is in flight at any time writes long contiguous runs.
+//               Measured on MI355X (float32 16384^2): square 64x64 tiles in
+//               column-fastest order 4.5 TB/s whether staged through LDS or
+//               registers; row-fastest order 5.4 TB/s; 256 x 64 tiles with
+//               non-temporal loads and stores 6.0 TB/s.  A tile that tall would
+//               need 64 KiB of LDS per workgroup; in registers it needs none.
+//               Non-temporal access only pays when every row starts on a 128-byte
+//               line (16384-wide float32: 6.0 vs 5.4 TB/s); when rows straddle
+//               lines it is far worse than cached access (16388-wide: 2.3 vs
+//               4.2 TB/s) because neighbouring packets no longer meet in L2, so the
+//               kernel is instantiated both ways and the host picks by alignment.
 //   * strided - everything else (records such as 28-byte items, element strides,
-//              negative strides): one lane per (item, chunk) with the output
-//              index fastest, so writes stay as dense as the layout allows.
+//               negative strides): one lane per (item, chunk) with the output
+//               index fastest, so writes stay as dense as the layout allows.
 //
 // HBM roofline: every item is read once and written once, 2*rows*cols*itemsize.
 #include "common.h"
@@ -30,80 +42,97 @@ template <> struct ItemOf<4> { using type = uint32_t; };
 template <> struct ItemOf<8> { using type = uint64_t; };
 template <> struct ItemOf<16> { using type = Item16; };
 
-// A 16-byte packet of items that is only guaranteed the alignment of one item.
-// Global memory accepts such accesses; the compiler still emits one dwordx4.
+// Sixteen bytes as a vector the compiler can load / store with one instruction,
+// non-temporally, at any item-aligned address (global memory accepts 128-bit
+// accesses that are only item-aligned).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <int E> struct __attribute__((packed, aligned(E))) Packet {
-    typename ItemOf<E>::type item[16 / E];
+    u32x4 v;
 };
 
-// Tile edge in items: 256-byte rows on both sides, capped so the tile fits LDS
-// comfortably for the narrow item sizes.
-template <int E> struct TileOf {
-    static constexpr int edge = (E == 1) ? 128 : (256 / E);
-};
+// Shape of the workgroup tile per item size: WR x WC wavefronts, REP wavefront
+// tiles stacked along the rows per wavefront.  A wavefront tile is 8V x 8V items.
+template <int E> struct ShapeOf;
+template <> struct ShapeOf<1> { static constexpr int WR = 4, WC = 1, REP = 1; };   // 512 x 128
+template <> struct ShapeOf<2> { static constexpr int WR = 4, WC = 1, REP = 1; };   // 256 x 64
+template <> struct ShapeOf<4> { static constexpr int WR = 2, WC = 2, REP = 4; };   // 256 x 64
+template <> struct ShapeOf<8> { static constexpr int WR = 2, WC = 2, REP = 4; };   // 128 x 32
+template <> struct ShapeOf<16> { static constexpr int WR = 2, WC = 2, REP = 4; };  //  64 x 16
 
-template <int E>
-__global__ __launch_bounds__(kThreads) void transpose_tiled(const char *__restrict__ in, char *__restrict__ out,
-                                                             int64_t rows, int64_t cols, int64_t in_s0,
-                                                             int64_t out_s0, int64_t tiles_c)
+template <int E, bool GUARD, bool NT>
+__device__ __forceinline__ void move_block(const char *__restrict__ in, char *__restrict__ out, int64_t rows,
+                                           int64_t cols, int64_t in_s0, int64_t out_s0, int64_t r0, int64_t c0)
 {
+    // lane's V x V block has its top-left item at in[r0, c0]
     using Item = typename ItemOf<E>::type;
-    using Pack = Packet<E>;
-    constexpr int V = 16 / E;            // items per 128-bit access
-    constexpr int T = TileOf<E>::edge;   // tile is T x T items
-    constexpr int PPR = T / V;           // packets per tile row
-    __shared__ Item tile[T][T + 1];
-
-    const int tid = threadIdx.x;
-    const int64_t tile_r = (int64_t)blockIdx.x / tiles_c;
-    const int64_t tile_c = (int64_t)blockIdx.x % tiles_c;
-    const int64_t r0 = tile_r * T;
-    const int64_t c0 = tile_c * T;
-
-    // in[r0 + r, c0 + p*V ... + V)  ->  tile[r][p*V ...]
-#pragma unroll 4
-    for (int idx = tid; idx < T * PPR; idx += kThreads) {
-        const int r = idx / PPR;
-        const int p = idx % PPR;
-        const int64_t gr = r0 + r;
-        const int64_t gc = c0 + (int64_t)p * V;
-        if (gr < rows) {
-            const char *src = in + gr * in_s0 + gc * E;
-            if (gc + V <= cols) {
-                Pack v = *reinterpret_cast<const Pack *>(src);
+    constexpr int V = 16 / E;
+    union Block {
+        u32x4 pk[V];
+        Item it[V][V];
+    };
+    Block a, b;
 #pragma unroll
-                for (int j = 0; j < V; ++j)
-                    tile[r][p * V + j] = v.item[j];
-            } else {
-                for (int j = 0; j < V; ++j)
-                    if (gc + j < cols)
-                        tile[r][p * V + j] = *reinterpret_cast<const Item *>(src + (int64_t)j * E);
-            }
+    for (int j = 0; j < V; ++j) {
+        const char *src = in + (r0 + j) * in_s0 + c0 * E;
+        if (!GUARD || (r0 + j < rows && c0 + V <= cols)) {
+            const Packet<E> *p = reinterpret_cast<const Packet<E> *>(src);
+            a.pk[j] = NT ? __builtin_nontemporal_load(&p->v) : p->v;
+        } else if (r0 + j < rows) {
+            for (int k = 0; k < V; ++k)
+                if (c0 + k < cols)
+                    a.it[j][k] = *reinterpret_cast<const Item *>(src + (int64_t)k * E);
         }
     }
-    __syncthreads();
-
-    // tile[p*V ...][c]  ->  out[c0 + c, r0 + p*V ... + V)
-#pragma unroll 4
-    for (int idx = tid; idx < T * PPR; idx += kThreads) {
-        const int c = idx / PPR;
-        const int p = idx % PPR;
-        const int64_t gc = c0 + c;              // output row
-        const int64_t gr = r0 + (int64_t)p * V;  // first output column
-        if (gc < cols) {
-            char *dst = out + gc * out_s0 + gr * E;
-            if (gr + V <= rows) {
-                Pack v;
 #pragma unroll
-                for (int j = 0; j < V; ++j)
-                    v.item[j] = tile[p * V + j][c];
-                *reinterpret_cast<Pack *>(dst) = v;
-            } else {
-                for (int j = 0; j < V; ++j)
-                    if (gr + j < rows)
-                        *reinterpret_cast<Item *>(dst + (int64_t)j * E) = tile[p * V + j][c];
-            }
+    for (int i = 0; i < V; ++i)
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+            b.it[i][j] = a.it[j][i];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        char *dst = out + (c0 + i) * out_s0 + r0 * E;
+        if (!GUARD || (c0 + i < cols && r0 + V <= rows)) {
+            Packet<E> *p = reinterpret_cast<Packet<E> *>(dst);
+            if (NT)
+                __builtin_nontemporal_store(b.pk[i], &p->v);
+            else
+                p->v = b.pk[i];
+        } else if (c0 + i < cols) {
+            for (int k = 0; k < V; ++k)
+                if (r0 + k < rows)
+                    *reinterpret_cast<Item *>(dst + (int64_t)k * E) = b.it[i][k];
         }
+    }
+}
+
+template <int E, bool NT>
+__global__ __launch_bounds__(64 * ShapeOf<E>::WR * ShapeOf<E>::WC) void transpose_packets(
+    const char *__restrict__ in, char *__restrict__ out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
+    int64_t tiles_r)
+{
+    constexpr int V = 16 / E;
+    constexpr int WT = 8 * V;  // wavefront tile edge, in items
+    constexpr int WR = ShapeOf<E>::WR, WC = ShapeOf<E>::WC, REP = ShapeOf<E>::REP;
+    constexpr int TR = WT * WR * REP, TC = WT * WC;
+
+    // consecutive workgroups go down the input rows = along the output rows
+    const int64_t tile_c = (int64_t)blockIdx.x / tiles_r;
+    const int64_t tile_r = (int64_t)blockIdx.x % tiles_r;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wr = wave / WC, wc = wave % WC;
+    const int cx = lane & 7, ry = lane >> 3;
+    const int64_t r_base = tile_r * TR + (int64_t)wr * (WT * REP) + ry * V;
+    const int64_t c0 = tile_c * TC + (int64_t)wc * WT + cx * V;
+
+    const bool inside = (tile_r + 1) * TR <= rows && (tile_c + 1) * TC <= cols;
+    if (inside) {
+#pragma unroll
+        for (int q = 0; q < REP; ++q)
+            move_block<E, false, NT>(in, out, rows, cols, in_s0, out_s0, r_base + q * WT, c0);
+    } else {
+        for (int q = 0; q < REP; ++q)
+            if (r_base + q * WT < rows && c0 < cols)
+                move_block<E, true, NT>(in, out, rows, cols, in_s0, out_s0, r_base + q * WT, c0);
     }
 }
 
@@ -128,17 +157,25 @@ __global__ __launch_bounds__(kThreads) void transpose_strided(const char *__rest
 }
 
 template <int E>
-int launch_tiled(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
-                 hipStream_t stream)
+int launch_packets(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
+                   hipStream_t stream)
 {
-    constexpr int T = TileOf<E>::edge;
-    const int64_t tiles_r = (rows + T - 1) / T;
-    const int64_t tiles_c = (cols + T - 1) / T;
+    constexpr int WT = 8 * (16 / E);
+    constexpr int TR = WT * ShapeOf<E>::WR * ShapeOf<E>::REP, TC = WT * ShapeOf<E>::WC;
+    const int64_t tiles_r = (rows + TR - 1) / TR;
+    const int64_t tiles_c = (cols + TC - 1) / TC;
     const int64_t tiles = tiles_r * tiles_c;
     if (tiles > 0x7fffffffLL)
         return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL((transpose_tiled<E>), dim3((unsigned)tiles), dim3(kThreads), 0, stream, (const char *)in,
-                       (char *)out, rows, cols, in_s0, out_s0, tiles_c);
+    // stream past the caches only if every row of both arrays starts on a 128-byte line
+    const uint64_t mix = (uint64_t)(uintptr_t)in | (uint64_t)(uintptr_t)out | (uint64_t)in_s0 | (uint64_t)out_s0;
+    const dim3 grid((unsigned)tiles), block(64 * ShapeOf<E>::WR * ShapeOf<E>::WC);
+    if (mix % 128 == 0)
+        hipLaunchKernelGGL((transpose_packets<E, true>), grid, block, 0, stream, (const char *)in, (char *)out, rows,
+                           cols, in_s0, out_s0, tiles_r);
+    else
+        hipLaunchKernelGGL((transpose_packets<E, false>), grid, block, 0, stream, (const char *)in, (char *)out, rows,
+                           cols, in_s0, out_s0, tiles_r);
     return nbh_launch_status();
 }
 
@@ -181,11 +218,11 @@ extern "C" int nbh_transpose(const void *in, void *out, int64_t rows, int64_t co
     const bool unit_inner = in_s1 == itemsize && out_s1 == itemsize && in_s0 > 0 && out_s0 > 0;
     if (unit_inner && g == itemsize) {  // item size is a power of two <= 16 and items are aligned
         switch (itemsize) {
-        case 1: return launch_tiled<1>(in, out, rows, cols, in_s0, out_s0, s);
-        case 2: return launch_tiled<2>(in, out, rows, cols, in_s0, out_s0, s);
-        case 4: return launch_tiled<4>(in, out, rows, cols, in_s0, out_s0, s);
-        case 8: return launch_tiled<8>(in, out, rows, cols, in_s0, out_s0, s);
-        case 16: return launch_tiled<16>(in, out, rows, cols, in_s0, out_s0, s);
+        case 1: return launch_packets<1>(in, out, rows, cols, in_s0, out_s0, s);
+        case 2: return launch_packets<2>(in, out, rows, cols, in_s0, out_s0, s);
+        case 4: return launch_packets<4>(in, out, rows, cols, in_s0, out_s0, s);
+        case 8: return launch_packets<8>(in, out, rows, cols, in_s0, out_s0, s);
+        case 16: return launch_packets<16>(in, out, rows, cols, in_s0, out_s0, s);
         default: break;
         }
     }
