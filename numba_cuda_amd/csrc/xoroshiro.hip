@@ -189,6 +189,7 @@ __global__ __launch_bounds__(kInitBlock) void init_states_kernel(uint64_t *__res
 
 struct UniformF32 {
     using value_type = float;
+    static constexpr bool kHeavy = false;
     static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1)
     {
         // one exact product in double, one rounding to float
@@ -197,6 +198,7 @@ struct UniformF32 {
 };
 struct UniformF64 {
     using value_type = double;
+    static constexpr bool kHeavy = false;
     static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1)
     {
         return (double)(next_d(s0, s1) >> 11) * (1.0 / 9007199254740992.0);
@@ -207,6 +209,7 @@ struct UniformF64 {
 // available stand-in for correctly rounded float32 routines.
 struct NormalF32 {
     using value_type = float;
+    static constexpr bool kHeavy = true;
     static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1)
     {
         const float u1 = UniformF32::draw(s0, s1);
@@ -222,6 +225,7 @@ struct NormalF32 {
 // float32 (so its result is a float32); the square root and cosine are float64.
 struct NormalF64 {
     using value_type = double;
+    static constexpr bool kHeavy = true;
     static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1)
     {
         const float u1 = UniformF32::draw(s0, s1);
@@ -236,18 +240,39 @@ struct NormalF64 {
 
 constexpr int kFillBlock = 256;
 
+// 16 bytes of output values that are only guaranteed the alignment of one value
+// (runs start at t*count, which need not be a multiple of four values).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <typename VT> struct __attribute__((packed, aligned(sizeof(VT)))) OutPacket {
+    u32x4 v;
+};
+
+// Each wavefront works on its own 64 generators and its own slice of LDS, so
+// wavefronts never wait for one another.  A round is 128 bytes per generator: the
+// lane draws them into registers, parks them in its LDS row with 128-bit writes
+// (row pitch 144 bytes keeps those conflict-free), and the wavefront then reads
+// the rows back eight lanes per row and stores 16 bytes per lane, so one store
+// instruction covers eight whole 128-byte lines.  Within a wavefront LDS accesses
+// execute in program order; the wavefront-scope fences only keep the compiler
+// from moving them across the hand-over.
 template <typename Gen>
 __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__ states, int64_t n,
                                                           typename Gen::value_type *__restrict__ out,
                                                           int64_t count)
 {
     using VT = typename Gen::value_type;
-    constexpr int ROUND = 128 / (int)sizeof(VT);  // one 128-byte line per generator per round
-    __shared__ VT park[kFillBlock][ROUND + 1];
+    constexpr int ROUND = 128 / (int)sizeof(VT);  // values per generator per round
+    constexpr int PER = 16 / (int)sizeof(VT);     // values per 16-byte packet
+    constexpr int PITCH = ROUND + PER;            // 144-byte rows
+    __shared__ __attribute__((aligned(16))) VT park_all[kFillBlock / 64][64][PITCH];
 
-    const int tid = threadIdx.x;
-    const int64_t t0 = (int64_t)blockIdx.x * kFillBlock;  // first generator of this workgroup
-    const int64_t t = t0 + tid;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    VT(*park)[PITCH] = park_all[wave];
+    const int64_t t0 = ((int64_t)blockIdx.x * (kFillBlock / 64) + wave) * 64;  // first generator of this wavefront
+    if (t0 >= n)
+        return;
+    const int64_t t = t0 + lane;
     const bool live = t < n;
     typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
     uint64_t s0 = 0, s1 = 0;
@@ -256,32 +281,55 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
         s0 = v.x;
         s1 = v.y;
     }
-    int64_t lanes_here = n - t0;  // generators this workgroup really has
-    if (lanes_here > kFillBlock)
-        lanes_here = kFillBlock;
+    const int lanes_here = (n - t0 > 64) ? 64 : (int)(n - t0);  // generators this wavefront really has
     VT *__restrict__ base = out + t0 * count;
+    const int sub = lane & 7;   // which packet of a row this lane stores
+    const int row = lane >> 3;  // which of eight rows per store instruction
 
     for (int64_t i0 = 0; i0 < count; i0 += ROUND) {
         const int m = (int)((count - i0 < ROUND) ? (count - i0) : ROUND);
-        if (live)
+        if (m == ROUND && !Gen::kHeavy) {
+            if (live) {
+                union {
+                    VT val[ROUND];
+                    u32x4 pk[8];
+                } mine;
+#pragma unroll
+                for (int j = 0; j < ROUND; ++j)
+                    mine.val[j] = Gen::draw(s0, s1);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    *reinterpret_cast<u32x4 *>(&park[lane][k * PER]) = mine.pk[k];
+            }
+        } else if (live) {
+            // transcendental-heavy draws stay in a rolled loop: unrolling sixteen
+            // inlined log/cos bodies only thrashes the instruction cache
+#pragma unroll 1
             for (int j = 0; j < m; ++j)
-                park[tid][j] = Gen::draw(s0, s1);
-        __syncthreads();
+                park[lane][j] = Gen::draw(s0, s1);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         if (m == ROUND) {
-#pragma unroll 4
-            for (int f = tid; f < kFillBlock * ROUND; f += kFillBlock) {
-                const int l = f / ROUND, j = f % ROUND;
-                if (l < lanes_here)
-                    base[(int64_t)l * count + i0 + j] = park[l][j];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int l = k * 8 + row;
+                if (l < lanes_here) {
+                    u32x4 v = *reinterpret_cast<const u32x4 *>(&park[l][sub * PER]);
+                    reinterpret_cast<OutPacket<VT> *>(base + (int64_t)l * count + i0 + sub * PER)->v = v;
+                }
             }
         } else {
-            for (int f = tid; f < kFillBlock * m; f += kFillBlock) {
+            for (int f = lane; f < 64 * m; f += 64) {
                 const int l = f / m, j = f % m;
                 if (l < lanes_here)
                     base[(int64_t)l * count + i0 + j] = park[l][j];
             }
         }
-        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
     if (live) {
         u64x2 v = {s0, s1};
