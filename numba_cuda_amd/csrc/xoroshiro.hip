@@ -120,14 +120,26 @@ int device_table(const U128 **out)
 
 // ---- device side ------------------------------------------------------------------
 
-__device__ __forceinline__ uint64_t rotl_d(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+// The generator step on 32-bit halves: 64-bit rotations and the shift are funnel
+// shifts of register pairs (v_alignbit_b32), two instructions each.
+__device__ __forceinline__ uint32_t funnel(uint32_t hi, uint32_t lo, int right)
+{
+    return __builtin_amdgcn_alignbit(hi, lo, right);  // bits [right, right + 32) of hi:lo
+}
 
 __device__ __forceinline__ uint64_t next_d(uint64_t &s0, uint64_t &s1)
 {
     const uint64_t r = s0 + s1;
-    const uint64_t t = s1 ^ s0;
-    s0 = rotl_d(s0, 55) ^ t ^ (t << 14);
-    s1 = rotl_d(t, 36);
+    const uint32_t a_lo = (uint32_t)s0, a_hi = (uint32_t)(s0 >> 32);
+    const uint32_t t_lo = a_lo ^ (uint32_t)s1, t_hi = a_hi ^ (uint32_t)(s1 >> 32);
+    // rotl(s0, 55): swap halves, then rotate left by 23
+    const uint32_t r55_hi = funnel(a_lo, a_hi, 9), r55_lo = funnel(a_hi, a_lo, 9);
+    // t << 14
+    const uint32_t sh_hi = funnel(t_hi, t_lo, 18), sh_lo = t_lo << 14;
+    // rotl(t, 36): swap halves, then rotate left by 4
+    const uint32_t r36_hi = funnel(t_lo, t_hi, 28), r36_lo = funnel(t_hi, t_lo, 28);
+    s0 = ((uint64_t)(r55_hi ^ t_hi ^ sh_hi) << 32) | (r55_lo ^ t_lo ^ sh_lo);
+    s1 = ((uint64_t)r36_hi << 32) | r36_lo;
     return r;
 }
 
@@ -187,22 +199,33 @@ __global__ __launch_bounds__(kInitBlock) void init_states_kernel(uint64_t *__res
 
 // ---- draws -------------------------------------------------------------------------
 
+// (x >> 11) * 2^-53 without integer-to-double conversions.  With m = x >> 11 =
+// hi * 2^32 + lo (hi < 2^21), the doubles whose bit patterns are
+//   {0x41E00000, hi} = 2^31 + hi * 2^-21      and      {0x3FE00000, lo} = 2^-1 + lo * 2^-53
+// carry the two halves in their mantissas; (first - (2^31 + 2^-1)) + second is
+// m * 2^-53, and both additions are exact (every intermediate is a multiple of
+// 2^-53 below 1 in magnitude).
+__device__ __forceinline__ double unit_double(uint64_t x)
+{
+    const uint64_t m = x >> 11;
+    const double a = __builtin_bit_cast(double, (uint64_t)0x41E0000000000000ull | (m >> 32));
+    const double b = __builtin_bit_cast(double, (uint64_t)0x3FE0000000000000ull | (m & 0xFFFFFFFFull));
+    return (a - 2147483648.5) + b;
+}
+
 struct UniformF32 {
     using value_type = float;
     static constexpr bool kHeavy = false;
     static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1)
     {
-        // one exact product in double, one rounding to float
-        return (float)((double)(next_d(s0, s1) >> 11) * (1.0 / 9007199254740992.0));
+        // the exact value in double, then one rounding to float
+        return (float)unit_double(next_d(s0, s1));
     }
 };
 struct UniformF64 {
     using value_type = double;
     static constexpr bool kHeavy = false;
-    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1)
-    {
-        return (double)(next_d(s0, s1) >> 11) * (1.0 / 9007199254740992.0);
-    }
+    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1) { return unit_double(next_d(s0, s1)); }
 };
 // Box-Muller, cosine branch.  The float32 variant works in float32 throughout;
 // log and cos are evaluated in double and rounded once, which is the closest
