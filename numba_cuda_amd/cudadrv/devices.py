@@ -79,6 +79,9 @@ class _Runtime:
         """Context of device `devnum` (None: the thread's current device, or
         device 0 when the thread has not chosen yet), made current."""
         if devnum is None:
+            ctx = getattr(self._tls, "ctx", None)
+            if ctx is not None:          # the common case: this thread already has a device
+                return ctx
             devnum = self.current_device
             if devnum is None:
                 devnum = 0
@@ -86,11 +89,13 @@ class _Runtime:
             device = driver.get_device(devnum)   # validates devnum
             driver.nbh_set_device(devnum)
             self._tls.devnum = devnum
+            self._tls.ctx = None
         else:
             device = driver.get_device(devnum)
         with self._lock:
             ctx = device.get_primary_context()
         ctx.prepare_for_use()
+        self._tls.ctx = ctx
         return ctx
 
     def reset(self):
@@ -98,6 +103,7 @@ class _Runtime:
         for dev in driver.list_devices() if driver.is_initialized and driver.lib else []:
             dev.reset()
         self._tls.devnum = None
+        self._tls.ctx = None
 
 
 _runtime = _Runtime()

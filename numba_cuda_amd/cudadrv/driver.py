@@ -535,22 +535,20 @@ class Context:
 
     _RESULT_SLOT_BYTES = 256
 
-    @property
-    def reduce_scratch_bytes(self):
-        return driver.lib.nbh_reduce_scratch_bytes()
-
     def reduce_scratch(self, stream_handle):
-        """(scratch memory, address of a result slot) for nbh_reduce on the given
-        stream, made and zeroed on first use.  Work on one stream is ordered, so
-        consecutive reductions on it can share both; different streams get their
-        own.  The slot sits behind the scratch area in the same allocation."""
-        mem = self._scratch.get(stream_handle)
-        if mem is None:
-            nbytes = self.reduce_scratch_bytes
+        """(scratch address, result slot address, scratch size) for nbh_reduce on
+        the given stream, made and zeroed on first use.  Work on one stream is
+        ordered, so consecutive reductions on it can share both; different streams
+        get their own.  The slot sits behind the scratch area in the same
+        allocation."""
+        entry = self._scratch.get(stream_handle)
+        if entry is None:
+            nbytes = driver.lib.nbh_reduce_scratch_bytes()
             mem = self.memalloc(nbytes + self._RESULT_SLOT_BYTES)
-            driver.nbh_memset8(mem.device_ctypes_pointer.value, 0, nbytes + self._RESULT_SLOT_BYTES, None)
-            self._scratch[stream_handle] = mem
-        return mem, mem.device_ctypes_pointer.value + self.reduce_scratch_bytes
+            ptr = mem.device_ctypes_pointer.value
+            driver.nbh_memset8(ptr, 0, nbytes + self._RESULT_SLOT_BYTES, None)
+            entry = self._scratch[stream_handle] = (ptr, ptr + nbytes, nbytes, mem)
+        return entry[0], entry[1], entry[2]
 
     def __repr__(self):
         return "<HIP context of device %d>" % self.device.id

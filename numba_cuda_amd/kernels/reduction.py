@@ -157,6 +157,7 @@ class Reduce:
                 self._cache[functor] = self._op
             except TypeError:
                 pass
+        self._opcode = _lib.OP_CODES[self._op]
 
     def __call__(self, arr, size=None, res=None, init=0, stream=0):
         """Full reduction of `arr`.
@@ -173,42 +174,71 @@ class Reduce:
             raise TypeError("only support 1D array")
         if size is not None:
             arr = arr[:size]
-        init = arr.dtype.type(init)
+        dtype = arr.dtype
         if arr.size < 1:
-            return init          # `res` is left untouched, as in the reference
+            return dtype.type(init)          # `res` is left untouched, as in the reference
 
-        code = _lib.DTYPE_CODES.get(arr.dtype.name)
-        if code is None or not arr.dtype.isnative:
-            raise NotImplementedError("Reduce does not support dtype %s" % arr.dtype)
+        code = _DTYPE_CODE.get(dtype)
+        if code is None:
+            raise NotImplementedError("Reduce does not support dtype %s" % dtype)
 
         ctx = devices.get_context()
         if not _driver.is_device_memory(arr):
             # host input: implicit transfer, as a kernel argument would get
             arr, _ = devicearray.auto_device(arr, stream=stream)
-        if arr.strides[0] != arr.dtype.itemsize:
+        if arr.strides[0] != dtype.itemsize:
             raise NotImplementedError("Reduce needs a unit-stride array; got strides %s" % (arr.strides,))
 
-        hstream = _driver._stream_handle(stream)
-        scratch, slot = ctx.reduce_scratch(hstream)
+        hstream = stream.handle if type(stream) is _driver.Stream else _driver._stream_handle(stream)
+        scratch_ptr, slot, scratch_bytes = ctx.reduce_scratch(hstream)
         if res is not None:
-            if res.dtype != arr.dtype:
-                raise TypeError("res has dtype %s, expected %s" % (res.dtype, arr.dtype))
+            if res.dtype != dtype:
+                raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
             out_ptr = res.device_ctypes_pointer.value
         else:
             out_ptr = slot      # per-stream result slot: no allocation per call
-        init_buf = np.array([init], dtype=arr.dtype)
-        _driver.driver.nbh_reduce(_lib.OP_CODES[self._op], code, arr.device_ctypes_pointer.value,
-                                  arr.size, init_buf.ctypes.data, out_ptr,
-                                  scratch.device_ctypes_pointer.value, ctx.reduce_scratch_bytes,
-                                  hstream or None)
+        init_ptr = _init_buffer(dtype, init)
+        drv = _driver.driver
+        rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size, init_ptr,
+                                out_ptr, scratch_ptr, scratch_bytes, hstream or None)
+        if rc:
+            drv.check("nbh_reduce", rc)
         if res is not None:
             return None
         # the value is wanted on the host now: wait for the stream, then fetch it
         if hstream:
-            _driver.driver.nbh_stream_synchronize(hstream)
-        host = np.empty(1, dtype=arr.dtype)
-        _driver.driver.nbh_memcpy_d2h(host.ctypes.data, out_ptr, arr.dtype.itemsize, None)
+            drv.nbh_stream_synchronize(hstream)
+        host = np.empty(1, dtype=dtype)
+        drv.nbh_memcpy_d2h(host.ctypes.data, out_ptr, dtype.itemsize, None)
         return host[0]
+
+
+_DTYPE_CODE = {np.dtype(name): code for name, code in _lib.DTYPE_CODES.items()}
+
+# host copies of `init` values, one element each, kept alive for the process:
+# (dtype, init) -> (array, address).  nbh_reduce reads the value during the call.
+_INIT_CACHE = {}
+
+
+def _init_buffer(dtype, init):
+    try:
+        return _INIT_CACHE[dtype, init][1]
+    except (KeyError, TypeError):
+        pass
+    buf = np.array([dtype.type(init)], dtype=dtype)
+    try:
+        if len(_INIT_CACHE) < 4096 and init == init:     # NaN never compares equal: do not cache it
+            _INIT_CACHE[dtype, init] = (buf, buf.ctypes.data)
+            return buf.ctypes.data
+    except TypeError:
+        pass
+    _KEEPALIVE.append(buf)
+    if len(_KEEPALIVE) > 64:
+        del _KEEPALIVE[:32]
+    return buf.ctypes.data
+
+
+_KEEPALIVE = []
 
 
 reduce = Reduce
