@@ -35,6 +35,10 @@ MEASURED_TRAFFIC = {
     "reduce_f32_sum": 1073811861,
     # profiles/copy_flat_f32_2p28.txt: the calibration kernel itself
     "copy_f32": 2147483648,
+    # profiles/transpose_packets_f32_16384sq.txt: 1 073 769 401 B fetched + 1 074 524 157 B written
+    "transpose_f32": 2148293558,
+    # profiles/xoroshiro_fill_and_init_2p24.txt: 268 534 300 B fetched + 4 563 402 098 B written
+    "rng_uniform_f32": 4831936398,
 }
 
 
