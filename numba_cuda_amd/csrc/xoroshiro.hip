@@ -4,9 +4,17 @@
 // State initialisation.  The reference builds states[i] = jump^i(states[0]) as one
 // sequential chain on the CPU.  `next` is linear over GF(2), so `jump` (2^64 steps)
 // is a 128x128 bit matrix J; the host tabulates J^(2^k), k = 0..63, once per
-// process, and lane l of a wavefront computes J^(base+l) * s by binary expansion of
-// the exponent (bits >= 6 are uniform across the wavefront), then keeps stepping by
-// J^64 so that each step of the wavefront writes 64 consecutive states (1 KiB).
+// process.  A wavefront owns 4096 consecutive states: lane l starts at
+// J^(first + l) * s and keeps stepping by J^64, so every step of the wavefront
+// writes 64 consecutive states (1 KiB).  Three kinds of matrix-vector product:
+//   * J^first (bits >= 12 of the index, the same vector in every lane): the 64
+//     lanes split the 128 columns between them and XOR-reduce across the
+//     wavefront - about 40 instructions per product instead of 1150;
+//   * J^l, l < 64 (a different matrix subset per lane) and the J^64 step (a
+//     different vector per lane): lookup tables in LDS, 4 bits of the vector per
+//     lookup for J^1..J^32 and 8 bits per lookup for J^64 (112 KiB per workgroup,
+//     one 1024-thread workgroup per compute unit);
+//   * small arrays skip the tables and use masked XORs over all 128 columns.
 //
 // Draws.  Each lane owns one generator whose 128-bit state stays in registers.
 // The reference's layout out[t*count + i] gives every lane its own run of `count`
@@ -53,9 +61,15 @@ inline U128 jump_h(U128 s)
 constexpr int kPowers = 64;
 // table[k][c] = column c of J^(2^k): the image of the state with only bit c set
 // (bits 0..63 live in s0, bits 64..127 in s1).
+constexpr int kLaneTables = 6;  // J^1 .. J^32, indexed by 4 bits of the vector
 struct JumpTable {
     U128 col[kPowers][128];
+    // lut4[k][p][v]: XOR of columns 4p+b of J^(2^k) over the set bits b of v
+    U128 lut4[kLaneTables][32][16];
+    // lut8[p][v]: XOR of columns 8p+b of J^64 over the set bits b of v
+    U128 lut8[16][256];
 };
+constexpr int kLutEntries = kLaneTables * 32 * 16 + 16 * 256;  // lut4 and lut8 are contiguous
 
 inline U128 apply_h(const U128 *m, U128 v)
 {
@@ -86,13 +100,34 @@ const JumpTable &jump_table()
         for (int k = 1; k < kPowers; ++k)  // square: column c of M*M is M applied to column c of M
             for (int c = 0; c < 128; ++c)
                 t->col[k][c] = apply_h(t->col[k - 1], t->col[k - 1][c]);
+        for (int k = 0; k < kLaneTables; ++k)
+            for (int p = 0; p < 32; ++p)
+                for (int v = 0; v < 16; ++v) {
+                    U128 x = {0, 0};
+                    for (int b = 0; b < 4; ++b)
+                        if ((v >> b) & 1) {
+                            x.s0 ^= t->col[k][4 * p + b].s0;
+                            x.s1 ^= t->col[k][4 * p + b].s1;
+                        }
+                    t->lut4[k][p][v] = x;
+                }
+        for (int p = 0; p < 16; ++p)
+            for (int v = 0; v < 256; ++v) {
+                U128 x = {0, 0};
+                for (int b = 0; b < 8; ++b)
+                    if ((v >> b) & 1) {
+                        x.s0 ^= t->col[6][8 * p + b].s0;
+                        x.s1 ^= t->col[6][8 * p + b].s1;
+                    }
+                t->lut8[p][v] = x;
+            }
         table = t;
     });
     return *table;
 }
 
 // Device copy of the table, one per device, made on first use and kept for the
-// life of the process (128 KiB).
+// life of the process (240 KiB: matrix columns and lookup tables).
 int device_table(const U128 **out)
 {
     constexpr int kMaxDev = 64;
@@ -194,6 +229,92 @@ __global__ __launch_bounds__(kInitBlock) void init_states_kernel(uint64_t *__res
         }
         if (g + 1 < kInitSteps)
             apply_d(step, s0, s1);
+    }
+}
+
+// XOR of a value over the 64 lanes, returned in every lane.
+__device__ __forceinline__ uint32_t wave_xor32(uint32_t v)
+{
+    v ^= (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0xB1, 0xF, 0xF, false);   // lane ^ 1
+    v ^= (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x4E, 0xF, 0xF, false);   // lane ^ 2
+    v ^= (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x141, 0xF, 0xF, false);  // other quad of 8
+    v ^= (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x140, 0xF, 0xF, false);  // other half of 16
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 0) ^ (uint32_t)__builtin_amdgcn_readlane((int)v, 16) ^
+           (uint32_t)__builtin_amdgcn_readlane((int)v, 32) ^ (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+}
+__device__ __forceinline__ uint64_t wave_xor64(uint64_t v)
+{
+    return ((uint64_t)wave_xor32((uint32_t)(v >> 32)) << 32) | wave_xor32((uint32_t)v);
+}
+
+// r = M * (s0, s1) when every lane holds the SAME vector: lane l contributes
+// columns l and 64 + l, the wavefront XORs the contributions together.
+__device__ __forceinline__ void apply_shared(const U128 *__restrict__ m, int lane, uint64_t &s0, uint64_t &s1)
+{
+    const U128 ca = m[lane], cb = m[64 + lane];
+    const uint64_t ma = 0 - ((s0 >> lane) & 1), mb = 0 - ((s1 >> lane) & 1);
+    const uint64_t p0 = (ca.s0 & ma) ^ (cb.s0 & mb);
+    const uint64_t p1 = (ca.s1 & ma) ^ (cb.s1 & mb);
+    s0 = wave_xor64(p0);
+    s1 = wave_xor64(p1);
+}
+
+typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
+
+// r = M * (s0, s1) from a table indexed by BITS bits of the vector at a time.
+template <int BITS>
+__device__ __forceinline__ void apply_lut(const u64x2_t *__restrict__ lut, uint64_t &s0, uint64_t &s1)
+{
+    constexpr int N = 1 << BITS;       // entries per position
+    constexpr int HALF = 64 / BITS;    // positions per 64-bit word
+    u64x2_t r = {0, 0};
+#pragma unroll
+    for (int p = 0; p < HALF; ++p) {
+        r ^= lut[p * N + (int)((s0 >> (p * BITS)) & (N - 1))];
+        r ^= lut[(HALF + p) * N + (int)((s1 >> (p * BITS)) & (N - 1))];
+    }
+    s0 = r.x;
+    s1 = r.y;
+}
+
+constexpr int kTabBlock = 1024;
+constexpr int64_t kTablesFrom = 1 << 18;  // below this the table load outweighs its benefit
+
+__global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t *__restrict__ states, int64_t n,
+                                                                       uint64_t b0, uint64_t b1,
+                                                                       const U128 *__restrict__ table,
+                                                                       const u64x2_t *__restrict__ lut_global)
+{
+    __shared__ u64x2_t lut[kLutEntries];  // 112 KiB: lut4[6][32][16] then lut8[16][256]
+    for (int i = threadIdx.x; i < kLutEntries; i += kTabBlock)
+        lut[i] = lut_global[i];
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kTabBlock / 64) + (threadIdx.x >> 6);
+    const int64_t first = wave * (64 * kInitSteps);
+    if (first >= n)
+        return;
+    uint64_t s0 = b0, s1 = b1;
+    const uint64_t hi = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 6)) |
+                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 38)) << 32);
+    for (int k = 6; k < kPowers; ++k)
+        if ((hi >> (k - 6)) & 1)
+            apply_shared(table + (size_t)k * 128, lane, s0, s1);
+    for (int k = 0; k < kLaneTables; ++k)
+        if ((lane >> k) & 1)
+            apply_lut<4>(lut + k * 32 * 16, s0, s1);
+    const u64x2_t *__restrict__ step = lut + kLaneTables * 32 * 16;  // J^64, 8 bits per lookup
+    for (int g = 0; g < kInitSteps; ++g) {
+        if (first + (int64_t)g * 64 >= n)
+            break;
+        const int64_t idx = first + (int64_t)g * 64 + lane;
+        if (idx < n) {
+            u64x2_t v = {s0, s1};
+            *reinterpret_cast<u64x2_t *>(states + 2 * idx) = v;
+        }
+        if (g + 1 < kInitSteps)
+            apply_lut<8>(step, s0, s1);
     }
 }
 
@@ -405,12 +526,22 @@ int nbh_xoro_init_states(void *states, int64_t n, uint64_t seed, uint64_t subseq
     int rc = device_table(&dtable);
     if (rc)
         return rc;
+    hipStream_t hs = nbh_hip_stream(stream);
+    if (n >= kTablesFrom) {
+        // one workgroup of 16 wavefronts per 65536 states, lookup tables in LDS
+        const int64_t per_block = (int64_t)(kTabBlock / 64) * 64 * kInitSteps;
+        const int64_t grid = (n + per_block - 1) / per_block;
+        if (grid > 0x7fffffffLL)
+            return (int)hipErrorInvalidValue;
+        const u64x2_t *lut = reinterpret_cast<const u64x2_t *>(dtable + (size_t)kPowers * 128);
+        hipLaunchKernelGGL(init_states_tables_kernel, dim3((unsigned)grid), dim3(kTabBlock), 0, hs,
+                           (uint64_t *)states, n, base.s0, base.s1, dtable, lut);
+        return nbh_launch_status();
+    }
     const int64_t per_block = (int64_t)(kInitBlock / 64) * 64 * kInitSteps;
     const int64_t grid = (n + per_block - 1) / per_block;
-    if (grid > 0x7fffffffLL)
-        return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL(init_states_kernel, dim3((unsigned)grid), dim3(kInitBlock), 0, nbh_hip_stream(stream),
-                       (uint64_t *)states, n, base.s0, base.s1, dtable);
+    hipLaunchKernelGGL(init_states_kernel, dim3((unsigned)grid), dim3(kInitBlock), 0, hs, (uint64_t *)states, n,
+                       base.s0, base.s1, dtable);
     return nbh_launch_status();
 }
 
