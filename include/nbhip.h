@@ -105,6 +105,11 @@ int nbh_stream_create(nbh_stream_t *stream);
 int nbh_stream_destroy(nbh_stream_t stream);
 int nbh_stream_synchronize(nbh_stream_t stream);
 int nbh_stream_query(nbh_stream_t stream);
+/* cudadrv/driver.py:1937-1973 Stream.add_callback (cuStreamAddCallback): `fn(user)`
+ * runs on a runtime thread once all work queued on `stream` so far has finished.
+ * No library call may be made from inside `fn`. */
+typedef void (*nbh_host_fn)(void *user);
+int nbh_stream_add_callback(nbh_stream_t stream, nbh_host_fn fn, void *user);
 /* cudadrv/driver.py:1273-1280 Context.create_event, :2037-2095 Event */
 int nbh_event_create(nbh_event_t *event, int timing);
 int nbh_event_destroy(nbh_event_t event);

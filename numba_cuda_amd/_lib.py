@@ -47,6 +47,7 @@ SIGNATURES = {
     "nbh_stream_destroy": (c_int, [c_vp]),
     "nbh_stream_synchronize": (c_int, [c_vp]),
     "nbh_stream_query": (c_int, [c_vp]),
+    "nbh_stream_add_callback": (c_int, [c_vp, ctypes.CFUNCTYPE(None, c_vp), c_vp]),
     "nbh_event_create": (c_int, [P(c_vp), c_int]),
     "nbh_event_destroy": (c_int, [c_vp]),
     "nbh_event_record": (c_int, [c_vp, c_vp]),
@@ -75,6 +76,8 @@ OP_CODES = {"add": 0, "mul": 1, "max": 2, "min": 3}
 HIP_SUCCESS = 0
 HIP_ERROR_OUT_OF_MEMORY = 2
 HIP_ERROR_NOT_READY = 600
+
+HOST_FN = ctypes.CFUNCTYPE(None, c_vp)
 
 _lib = None
 

@@ -189,6 +189,13 @@ int nbh_stream_destroy(nbh_stream_t stream) { return (int)hipStreamDestroy(nbh_h
 int nbh_stream_synchronize(nbh_stream_t stream) { return (int)hipStreamSynchronize(nbh_hip_stream(stream)); }
 int nbh_stream_query(nbh_stream_t stream) { return (int)hipStreamQuery(nbh_hip_stream(stream)); }
 
+int nbh_stream_add_callback(nbh_stream_t stream, nbh_host_fn fn, void *user)
+{
+    if (!fn)
+        return (int)hipErrorInvalidValue;
+    return (int)hipLaunchHostFunc(nbh_hip_stream(stream), fn, user);
+}
+
 int nbh_event_create(nbh_event_t *event, int timing)
 {
     if (!event)

@@ -843,6 +843,53 @@ class Stream:
         yield self
         self.synchronize()
 
+    def add_callback(self, callback, arg=None):
+        """Call `callback(stream, status, arg)` from a runtime thread once everything
+        queued on this stream so far has finished (status is 0).  The callback must
+        not call back into the GPU API and should be short: later work on the stream
+        waits for it."""
+        token = object()
+
+        def trampoline(_user):
+            try:
+                callback(self, 0, arg)
+            except Exception as e:   # nothing can propagate out of a runtime thread
+                import warnings
+                warnings.warn("Exception in stream callback: %s" % (e,))
+            finally:
+                _live_callbacks.pop(token, None)
+
+        cfn = _lib.HOST_FN(trampoline)
+        _live_callbacks[token] = cfn          # keep the thunk alive until it has run
+        try:
+            driver.nbh_stream_add_callback(self.handle or None, cfn, None)
+        except Exception:
+            _live_callbacks.pop(token, None)
+            raise
+
+    def async_done(self):
+        """Awaitable that resolves (to this stream) once all work queued so far is done."""
+        import asyncio
+        loop = asyncio.get_running_loop()
+        future = loop.create_future()
+
+        def resolver(fut, status):
+            if fut.done():
+                return
+            if status == 0:
+                fut.set_result(self)
+            else:
+                fut.set_exception(Exception("Stream error %s" % status))
+
+        def callback(stream, status, fut):
+            loop.call_soon_threadsafe(resolver, fut, status)
+
+        self.add_callback(callback, future)
+        return future
+
+
+_live_callbacks = {}
+
 
 def _query(code, fname):
     if code == _lib.HIP_ERROR_NOT_READY:

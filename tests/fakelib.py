@@ -183,6 +183,32 @@ class FakeLib:
     def nbh_stream_query(self, s):
         return 0
 
+    def nbh_stream_add_callback(self, s, fn, user):
+        fn(user)                       # nothing is ever pending on the fake
+        return 0
+
+    def nbh_assign(self, dst, src, ndim, shape, dst_strides, src_strides, itemsize, stream):
+        """Strided broadcast assignment done with NumPy over raw host memory."""
+        import numpy as np
+        from numpy.lib.stride_tricks import as_strided
+        self._log("assign", _addr(dst), _addr(src), ndim, _addr(stream))
+        shp = tuple(shape[i] for i in range(ndim))
+        ds = tuple(dst_strides[i] for i in range(ndim))
+        ss = tuple(src_strides[i] for i in range(ndim))
+        if any(n == 0 for n in shp):
+            return 0
+        item = np.dtype((np.void, int(itemsize)))
+
+        def view(addr, strides):
+            lo = sum(min(0, (n - 1) * st) for n, st in zip(shp, strides))
+            hi = sum(max(0, (n - 1) * st) for n, st in zip(shp, strides)) + int(itemsize)
+            raw = (ctypes.c_ubyte * (hi - lo)).from_address(addr + lo)
+            base = np.frombuffer(raw, dtype=np.uint8)
+            return as_strided(base[-lo:-lo + int(itemsize)].view(item), shape=shp, strides=strides)
+
+        view(_addr(dst), ds)[...] = view(_addr(src), ss)
+        return 0
+
     def nbh_event_create(self, out, timing):
         h = self._handle()
         self.live_events.add(h)

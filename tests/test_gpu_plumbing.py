@@ -102,3 +102,28 @@ def test_setitem_scalars_rows_columns_broadcast():
     np.testing.assert_array_equal(t.copy_to_host(), big)
     t[1:] = cuda.to_device(big)[:-1]                 # misaligned flat copy
     np.testing.assert_array_equal(t.copy_to_host()[1:], big[:-1])
+
+
+def test_stream_callback_and_async_done():
+    import asyncio
+    import threading
+    s = cuda.stream()
+    a = cuda.to_device(np.arange(1 << 20, dtype=np.float32), stream=s)
+    done = threading.Event()
+    seen = []
+
+    def cb(stream, status, arg):
+        seen.append((stream is s, status, arg))
+        done.set()
+
+    out = cuda.device_array(1, np.float32)
+    cuda.reduce(lambda x, y: x + y)(a, res=out, stream=s)
+    s.add_callback(cb, "tag")
+    assert done.wait(10)
+    assert seen == [(True, 0, "tag")]
+
+    async def wait():
+        return await s.async_done()
+
+    assert asyncio.run(wait()) is s
+    assert abs(float(out[0]) - float(np.arange(1 << 20, dtype=np.float64).sum())) <= 2 * (1 << 20) * 6e-8 * 5.5e11

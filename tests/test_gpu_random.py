@@ -176,3 +176,31 @@ def test_config4_uniform_float32_2_pow_30_and_normal_float64():
         assert after[lo:lo + chunk].tobytes() == want_states.tobytes(), lo
     _say("normal_f64 worst ulp", worst)
     assert worst <= 2.0
+
+
+def test_normals_over_every_float32_mantissa_of_u1():
+    """The logarithm is the sensitive step of Box-Muller: a one-ulp float32
+    difference in log(u1) moves a float64 normal by ~2^28 ulp.  Sweep u1 over every
+    24-bit mantissa of two binades (crafted states whose first draw is chosen) and
+    require the usual 2 ulp against the oracle for both variants."""
+    n = 1 << 23
+    mant = np.arange(n, dtype=np.uint64)
+    rng = np.random.default_rng(11)
+    for top in (np.uint64(1) << np.uint64(63), np.uint64(1) << np.uint64(62)):
+        # first draw = s0 + s1; u1 = float32((draw >> 11) * 2^-53): put the mantissa
+        # just below the leading bit, random low bits
+        draw = top | (mant << np.uint64(40 if top >> np.uint64(63) else 39)) | \
+            rng.integers(0, 1 << 30, n, dtype=np.uint64)
+        st = np.zeros(n, nrandom.xoroshiro128p_dtype)
+        st["s1"] = rng.integers(0, 2**63, n, dtype=np.uint64)
+        st["s0"] = draw - st["s1"]
+        for kind, dtype in (("normal_f32", np.float32), ("normal_f64", np.float64)):
+            d = cuda.to_device(st)
+            out = cuda.device_array(n, dtype)
+            nrandom.xoroshiro128p_fill(d, out, 1, nrandom.NORMAL)
+            want, want_states = cref.fill(st, 1, kind)
+            got = out.copy_to_host()
+            u = _ulps(got, want)
+            _say(kind, "binade", int(top).bit_length(), "worst ulp", u.max(), "mismatching", int((u > 0).sum()))
+            assert u.max() <= 2.0
+            np.testing.assert_array_equal(d.copy_to_host(), want_states)

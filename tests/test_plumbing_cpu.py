@@ -116,3 +116,115 @@ def test_device_states_are_refused_by_scalar_functions(fake_gpu):
         nrandom.xoroshiro128p_uniform_float32(d, 0)
     with pytest.raises(TypeError, match="device array"):
         nrandom.xoroshiro128p_fill(np.zeros(4, nrandom.xoroshiro128p_dtype), d)
+
+
+def test_setitem_host_logic_and_synchronisation(fake_gpu):
+    """`darr[key] = value`: broadcasting rules, error messages and when the call
+    waits (reference: tests/cudadrv/test_cuda_array_slicing.py:220-379).  The fake
+    library performs the strided assignment with NumPy."""
+    a = np.arange(5 * 7, dtype=np.float64).reshape(5, 7)
+    d = cuda.to_device(a)
+    fake_gpu.calls.clear()
+    d[2, 3] = 500                       # no stream anywhere: default stream + wait
+    assert [c[0] for c in fake_gpu.calls if c[0] in ("assign", "stream_sync")][-2:] == ["assign", "stream_sync"]
+    a[2, 3] = 500
+    d[:, 2] = np.arange(5.0)
+    a[:, 2] = np.arange(5.0)
+    d[1:3] = np.array([[1.0], [2.0]])   # unit axis on the right repeats
+    a[1:3] = np.array([[1.0], [2.0]])
+    d[4] = 7
+    a[4] = 7
+    np.testing.assert_array_equal(d.copy_to_host(), a)
+    s = cuda.stream()
+    fake_gpu.calls.clear()
+    d.setitem(0, 1.5, stream=s)         # explicit stream: asynchronous, no wait
+    d.bind(s)[1] = 2.5                  # bound stream: asynchronous too
+    kinds = [c[0] for c in fake_gpu.calls if c[0] in ("assign", "stream_sync")]
+    assert kinds == ["assign", "assign"]
+    assert all(c[4] == int(s) for c in fake_gpu.calls if c[0] == "assign")
+    with pytest.raises(ValueError, match="Can't assign 3-D array to 2-D self"):
+        d[:] = np.zeros((1, 5, 7))
+    with pytest.raises(ValueError, match="Can't copy sequence with size 3 to array axis 1 with dimension 7"):
+        d[:] = np.zeros((5, 3))
+    with pytest.raises(TypeError, match="incompatible dtype"):
+        d[:] = cuda.to_device(np.zeros((5, 7), np.float32))
+
+
+def test_stream_callbacks(fake_gpu):
+    import asyncio
+    s = cuda.stream()
+    seen = []
+    s.add_callback(lambda stream, status, arg: seen.append((stream is s, status, arg)), "payload")
+    assert seen == [(True, 0, "payload")]
+    with pytest.warns(UserWarning, match="Exception in stream callback"):
+        s.add_callback(lambda *a: 1 / 0)
+
+    async def wait():
+        return await s.async_done()
+
+    assert asyncio.run(wait()) is s
+
+
+class _RecordingManager(cuda.HostOnlyCUDAMemoryManager):
+    """An External Memory Management plugin that only takes over device
+    allocations (the shape of the reference's tests/cudadrv/test_emm_plugins.py
+    :14-60 DeviceOnlyEMMPlugin)."""
+
+    log = []
+
+    def initialize(self):
+        self.log.append("initialize")
+
+    def memalloc(self, size):
+        import ctypes
+        from numba_cuda_amd.cudadrv import driver as drv
+        buf = ctypes.create_string_buffer(size)
+        self.log.append(("memalloc", size))
+        key = ctypes.addressof(buf)
+
+        def finalizer():
+            self.log.append(("free", size))
+            self.allocations.pop(key, None)
+
+        mem = drv.AutoFreePointer(self.context, key, size, finalizer=finalizer)
+        self.allocations[key] = (mem, buf)      # the manager keeps the pointer object alive
+        return mem.own()
+
+    def get_ipc_handle(self, memory):
+        raise NotImplementedError
+
+    def get_memory_info(self):
+        self.log.append("get_memory_info")
+        return cuda.MemoryInfo(free=32, total=64)
+
+    @property
+    def interface_version(self):
+        return 1
+
+
+def test_external_memory_manager_plugin(fake_gpu):
+    import gc
+    from numba_cuda_amd.cudadrv import driver as drv
+    _RecordingManager.log.clear()
+    cuda.set_memory_manager(_RecordingManager)
+    try:
+        ctx = cuda.current_context()
+        assert isinstance(ctx.memory_manager, _RecordingManager)
+        d = cuda.to_device(np.arange(10, dtype=np.int32))
+        assert ("memalloc", 40) in _RecordingManager.log
+        assert not any(c[0] == "malloc" for c in fake_gpu.calls)      # the default allocator is bypassed
+        np.testing.assert_array_equal(d.copy_to_host(), np.arange(10))
+        assert ctx.get_memory_info() == (32, 64)
+        del d
+        gc.collect()
+        assert ("free", 40) in _RecordingManager.log
+
+        class Wrong(_RecordingManager):
+            @property
+            def interface_version(self):
+                return 2
+
+        with pytest.raises(RuntimeError, match="EMM Plugin interface has version 2 - version 1 required"):
+            cuda.set_memory_manager(Wrong)
+    finally:
+        drv._memory_manager = None
