@@ -1,5 +1,10 @@
-"""The host API exported as `numba_cuda_amd.*` (reference:
-numba_cuda/numba/cuda/api.py:24-591)."""
+"""The host API exported as `numba_cuda_amd.*`.
+
+Same names, arguments and behaviour as numba_cuda/numba/cuda/api.py:24-591
+(arrays :24-168, :211-259, :290-374; streams and events :378-481; devices
+:484-567; defer_cleanup :570-586).  Every function that touches the GPU first makes
+sure the calling thread has a device selected.
+"""
 
 import contextlib
 
@@ -14,195 +19,222 @@ current_context = devices.get_context
 gpus = devices.gpus
 
 
-# ---- arrays ------------------------------------------------------------------------
+def _ctx():
+    return devices.get_context()
 
-@require_context
+
+# ---- device arrays ---------------------------------------------------------------------
+
+def device_array(shape, dtype=np.float64, strides=None, order="C", stream=0):
+    """Uninitialised device array, like numpy.empty."""
+    _ctx()
+    shape, strides, dtype = prepare_shape_strides_dtype(shape, strides, dtype, order)
+    return devicearray.DeviceNDArray(shape=shape, strides=strides, dtype=dtype, stream=stream)
+
+
+def to_device(obj, stream=0, copy=True, to=None):
+    """Allocate a device array like `obj` and copy `obj` into it; with `to=` copy
+    into that existing device array instead.  Asynchronous iff `stream` is non-zero.
+
+        d_ary = cuda.to_device(ary)               # host -> device
+        hary = d_ary.copy_to_host()               # and back
+        d_ary.copy_to_host(ary, stream=stream)    # into an existing array, on a stream
+    """
+    _ctx()
+    if to is not None:
+        if copy:
+            to.copy_to_device(obj, stream=stream)
+        return to
+    return devicearray.auto_device(obj, stream=stream, copy=copy, user_explicit=True)[0]
+
+
+def _layout_like(ary):
+    """(strides, order) that give a compact array with `ary`'s shape and axis
+    ordering; strides is None when plain C / F order already does."""
+    order = "F" if ary.flags["F_CONTIGUOUS"] and not ary.flags["C_CONTIGUOUS"] else "C"
+    return _contiguous_strides_like_array(ary), order
+
+
+def _contiguous_strides_like_array(ary):
+    if ary.ndim <= 1 or ary.flags["C_CONTIGUOUS"] or ary.flags["F_CONTIGUOUS"]:
+        return None
+    # rank the axes by stride (stable), then lay them out in that order, innermost first
+    strides = [0] * ary.ndim
+    step = ary.dtype.itemsize
+    for axis in sorted(range(ary.ndim), key=lambda k: ary.strides[k]):
+        strides[axis] = step
+        step *= ary.shape[axis]
+    return tuple(strides)
+
+
+def _order_like_array(ary):
+    return _layout_like(ary)[1]
+
+
+def device_array_like(ary, stream=0):
+    strides, order = _layout_like(ary)
+    return device_array(shape=ary.shape, dtype=ary.dtype, strides=strides, order=order, stream=stream)
+
+
+def _pinned_ndarray(shape, dtype, strides, order, **alloc_flags):
+    """(ndarray over fresh page-locked host memory, the memory object)"""
+    shape, strides, dtype = prepare_shape_strides_dtype(shape, strides, dtype, order)
+    nbytes = driver.memory_size_from_info(shape, strides, dtype.itemsize)
+    mem = _ctx().memhostalloc(nbytes, **alloc_flags)
+    ary = np.ndarray(shape=shape, strides=strides, dtype=dtype, order=order, buffer=mem.as_buffer())
+    return ary, mem
+
+
+def pinned_array(shape, dtype=np.float64, strides=None, order="C"):
+    """Host ndarray in page-locked memory, like numpy.empty; copies to and from it
+    can be truly asynchronous."""
+    return _pinned_ndarray(shape, dtype, strides, order)[0]
+
+
+def pinned_array_like(ary):
+    strides, order = _layout_like(ary)
+    return pinned_array(shape=ary.shape, dtype=ary.dtype, strides=strides, order=order)
+
+
+def mapped_array(shape, dtype=np.float64, strides=None, order="C", stream=0, portable=False, wc=False):
+    """Host ndarray in page-locked memory that is also mapped into the device's
+    address space; usable wherever a device array is.  `portable`: usable from
+    every device; `wc`: write-combined (fast to write from the host, slow to read)."""
+    ary, mem = _pinned_ndarray(shape, dtype, strides, order, mapped=True, portable=portable, wc=wc)
+    out = np.ndarray.view(ary, type=devicearray.MappedNDArray)
+    out.device_setup(mem, stream=stream)
+    return out
+
+
+def mapped_array_like(ary, stream=0, portable=False, wc=False):
+    strides, order = _layout_like(ary)
+    return mapped_array(shape=ary.shape, dtype=ary.dtype, strides=strides, order=order, stream=stream,
+                        portable=portable, wc=wc)
+
+
 def from_cuda_array_interface(desc, owner=None, sync=True):
     """Wrap the memory described by a __cuda_array_interface__ dict in a
     DeviceNDArray without copying; `owner` is kept alive by the result.  If the
     description carries a stream and `sync` is true, that stream is synchronised
     first (switch off globally with NUMBA_CUDA_ARRAY_INTERFACE_SYNC=0)."""
-    version = desc.get("version")
-    if 1 <= version and desc.get("mask") is not None:
+    ctx = _ctx()
+    if desc.get("version") >= 1 and desc.get("mask") is not None:
         raise NotImplementedError("Masked arrays are not supported")
-    shape, strides, dtype = prepare_shape_strides_dtype(
-        desc["shape"], desc.get("strides"), desc["typestr"], order="C")
-    size = driver.memory_size_from_info(shape, strides, dtype.itemsize)
-    data = driver.MemoryPointer(current_context(), desc["data"][0], size=size, owner=owner)
-    stream_ptr = desc.get("stream", None)
-    if stream_ptr is not None:
-        stream = external_stream(stream_ptr)
+    shape, strides, dtype = prepare_shape_strides_dtype(desc["shape"], desc.get("strides"),
+                                                        desc["typestr"], order="C")
+    nbytes = driver.memory_size_from_info(shape, strides, dtype.itemsize)
+    mem = driver.MemoryPointer(ctx, desc["data"][0], size=nbytes, owner=owner)
+    stream = 0
+    foreign = desc.get("stream", None)
+    if foreign is not None:
+        stream = external_stream(foreign)
         if sync and config.CUDA_ARRAY_INTERFACE_SYNC:
             stream.synchronize()
-    else:
-        stream = 0
-    return devicearray.DeviceNDArray(shape=shape, strides=strides, dtype=dtype, gpu_data=data,
-                                     stream=stream)
+    return devicearray.DeviceNDArray(shape=shape, strides=strides, dtype=dtype, gpu_data=mem, stream=stream)
 
 
 def as_cuda_array(obj, sync=True):
     """View any object exporting __cuda_array_interface__ as a DeviceNDArray."""
-    interface = getattr(obj, "__cuda_array_interface__", None)
-    if interface is None:
+    if not is_cuda_array(obj):
         raise TypeError("*obj* doesn't implement the cuda array interface.")
-    return from_cuda_array_interface(interface, owner=obj, sync=sync)
+    return from_cuda_array_interface(obj.__cuda_array_interface__, owner=obj, sync=sync)
 
 
 def is_cuda_array(obj):
+    """True if `obj` exports __cuda_array_interface__ (its validity is not checked)."""
     return hasattr(obj, "__cuda_array_interface__")
 
 
-@require_context
-def to_device(obj, stream=0, copy=True, to=None):
-    """Allocate a device array like `obj` and copy `obj` into it; with `to=` copy
-    into an existing device array instead.  Asynchronous iff `stream` is non-zero."""
-    if to is None:
-        to, _ = devicearray.auto_device(obj, stream=stream, copy=copy, user_explicit=True)
-        return to
-    if copy:
-        to.copy_to_device(obj, stream=stream)
-    return to
-
-
-@require_context
-def device_array(shape, dtype=np.float64, strides=None, order="C", stream=0):
-    """Uninitialised device array, like numpy.empty."""
-    shape, strides, dtype = prepare_shape_strides_dtype(shape, strides, dtype, order)
-    return devicearray.DeviceNDArray(shape=shape, strides=strides, dtype=dtype, stream=stream)
-
-
-@require_context
-def pinned_array(shape, dtype=np.float64, strides=None, order="C"):
-    """Host ndarray in page-locked memory, like numpy.empty."""
-    shape, strides, dtype = prepare_shape_strides_dtype(shape, strides, dtype, order)
-    bytesize = driver.memory_size_from_info(shape, strides, dtype.itemsize)
-    mem = current_context().memhostalloc(bytesize)
-    return np.ndarray(shape=shape, strides=strides, dtype=dtype, order=order, buffer=mem.as_buffer())
-
-
-@require_context
-def mapped_array(shape, dtype=np.float64, strides=None, order="C", stream=0, portable=False, wc=False):
-    """Host ndarray in page-locked memory that is also mapped into the device's
-    address space; usable wherever a device array is."""
-    shape, strides, dtype = prepare_shape_strides_dtype(shape, strides, dtype, order)
-    bytesize = driver.memory_size_from_info(shape, strides, dtype.itemsize)
-    mem = current_context().memhostalloc(bytesize, mapped=True, portable=portable, wc=wc)
-    npary = np.ndarray(shape=shape, strides=strides, dtype=dtype, order=order, buffer=mem.as_buffer())
-    mappedview = np.ndarray.view(npary, type=devicearray.MappedNDArray)
-    mappedview.device_setup(mem, stream=stream)
-    return mappedview
-
-
-def synchronize():
-    "Wait for all work on the current device."
-    return current_context().synchronize()
-
-
-def _contiguous_strides_like_array(ary):
-    """Strides of a compact array with `ary`'s shape and axis ordering, or None if
-    plain C / F strides already do."""
-    if ary.flags["C_CONTIGUOUS"] or ary.flags["F_CONTIGUOUS"] or ary.ndim <= 1:
-        return None
-    # rank axes by stride (stable), then lay them out in that order, innermost first
-    ranked = sorted(range(ary.ndim), key=lambda k: ary.strides[k])
-    strides = [0] * ary.ndim
-    step = ary.dtype.itemsize
-    for k in ranked:
-        strides[k] = step
-        step *= ary.shape[k]
-    return tuple(strides)
-
-
-def _order_like_array(ary):
-    return "F" if ary.flags["F_CONTIGUOUS"] and not ary.flags["C_CONTIGUOUS"] else "C"
-
-
-def device_array_like(ary, stream=0):
-    return device_array(shape=ary.shape, dtype=ary.dtype, strides=_contiguous_strides_like_array(ary),
-                        order=_order_like_array(ary), stream=stream)
-
-
-def mapped_array_like(ary, stream=0, portable=False, wc=False):
-    return mapped_array(shape=ary.shape, dtype=ary.dtype, strides=_contiguous_strides_like_array(ary),
-                        order=_order_like_array(ary), stream=stream, portable=portable, wc=wc)
-
-
-def pinned_array_like(ary):
-    return pinned_array(shape=ary.shape, dtype=ary.dtype, strides=_contiguous_strides_like_array(ary),
-                        order=_order_like_array(ary))
-
-
-# ---- streams and events --------------------------------------------------------------
-
-@require_context
-def stream():
-    "A new stream (it synchronises with the default stream, as CUDA's default flags do)."
-    return current_context().create_stream()
-
-
-@require_context
-def default_stream():
-    return current_context().get_default_stream()
-
-
-@require_context
-def legacy_default_stream():
-    return current_context().get_legacy_default_stream()
-
-
-@require_context
-def per_thread_default_stream():
-    return current_context().get_per_thread_default_stream()
-
-
-@require_context
-def external_stream(ptr):
-    "Wrap a hipStream_t created elsewhere, given as an int."
-    return current_context().create_external_stream(ptr)
-
-
-@require_context
 @contextlib.contextmanager
 def pinned(*arylist):
     "Temporarily page-lock the host arrays in `arylist`."
-    pmlist = []
-    for ary in arylist:
-        pmlist.append(current_context().mempin(ary, driver.host_pointer(ary),
-                                               driver.host_memory_size(ary), mapped=False))
+    ctx = _ctx()
+    locks = [ctx.mempin(a, driver.host_pointer(a), driver.host_memory_size(a), mapped=False) for a in arylist]
     yield
-    del pmlist
+    del locks
 
 
-@require_context
 @contextlib.contextmanager
 def mapped(*arylist, **kws):
     "Temporarily page-lock and device-map the host arrays; yields device arrays."
     assert not kws or "stream" in kws, "Only accept 'stream' as keyword."
+    ctx = _ctx()
     stream = kws.get("stream", 0)
-    pmlist, devarylist = [], []
-    for ary in arylist:
-        pm = current_context().mempin(ary, driver.host_pointer(ary), driver.host_memory_size(ary),
-                                      mapped=True)
-        pmlist.append(pm)
-        devarylist.append(devicearray.from_array_like(ary, gpu_data=pm, stream=stream))
+    locks = [ctx.mempin(a, driver.host_pointer(a), driver.host_memory_size(a), mapped=True) for a in arylist]
+    views = [devicearray.from_array_like(a, gpu_data=lock, stream=stream) for a, lock in zip(arylist, locks)]
     try:
-        yield devarylist[0] if len(devarylist) == 1 else devarylist
+        yield views[0] if len(views) == 1 else views
     finally:
         # the caller's name for the yielded array outlives the with-block, so
         # unmapping cannot wait for reference counts
-        for pm in pmlist:
-            pm.free()
+        for lock in locks:
+            lock.free()
+
+
+# ---- streams, events, synchronisation ------------------------------------------------------
+
+def synchronize():
+    "Wait for all work on the current device."
+    return _ctx().synchronize()
+
+
+def stream():
+    "A new stream (it synchronises with the default stream, as CUDA's default flags do)."
+    return _ctx().create_stream()
+
+
+def default_stream():
+    "The default stream; in this API that is always the legacy (synchronising) one."
+    return _ctx().get_default_stream()
+
+
+def legacy_default_stream():
+    return _ctx().get_legacy_default_stream()
+
+
+def per_thread_default_stream():
+    return _ctx().get_per_thread_default_stream()
+
+
+def external_stream(ptr):
+    "Wrap a hipStream_t created elsewhere, given as an int."
+    return _ctx().create_external_stream(ptr)
 
 
 def event(timing=True):
     "A new event; `timing=False` makes it cheaper but unusable with elapsed_time."
-    return current_context().create_event(timing=timing)
+    return _ctx().create_event(timing=timing)
 
 
 event_elapsed_time = driver.event_elapsed_time
 
 
-# ---- devices ------------------------------------------------------------------------
+@contextlib.contextmanager
+def defer_cleanup():
+    """Hold every deallocation off until the (outermost) block exits, so that no free
+    interrupts asynchronous work issued inside it."""
+    with _ctx().defer_cleanup():
+        yield
+
+
+def profile_start():
+    _ctx()
+    driver.profile_start()
+
+
+def profile_stop():
+    _ctx()
+    driver.profile_stop()
+
+
+@contextlib.contextmanager
+def profiling():
+    profile_start()
+    yield
+    profile_stop()
+
+
+# ---- devices ----------------------------------------------------------------------------------
 
 def select_device(device_id):
     "Make `device_id` the calling thread's device; returns the Device."
@@ -210,7 +242,7 @@ def select_device(device_id):
 
 
 def get_current_device():
-    return current_context().device
+    return _ctx().device
 
 
 def list_devices():
@@ -224,31 +256,20 @@ def close():
 
 def detect():
     "Print a summary of the GPUs found; returns True if any is supported."
-    devlist = list_devices()
-    print("Found %d HIP devices" % len(devlist))
-    supported = 0
-    for dev in devlist:
+    found = list_devices()
+    print("Found %d HIP devices" % len(found))
+    usable = 0
+    for dev in found:
         ok = dev.WARP_SIZE == 64
-        supported += ok
+        usable += ok
         print("id %d    %20s %40s" % (dev.id, dev.name, "[SUPPORTED]" if ok else "[NOT SUPPORTED: needs wave64]"))
-        for key, val in (("Compute units", dev.MULTIPROCESSOR_COUNT), ("PCI Device ID", dev.PCI_DEVICE_ID),
-                         ("PCI Bus ID", dev.PCI_BUS_ID), ("Wavefront size", dev.WARP_SIZE)):
+        facts = {"Compute units": dev.MULTIPROCESSOR_COUNT, "PCI Device ID": dev.PCI_DEVICE_ID,
+                 "PCI Bus ID": dev.PCI_BUS_ID, "Wavefront size": dev.WARP_SIZE}
+        for key, val in facts.items():
             print("%40s: %s" % (key, val))
     print("Summary:")
-    print("\t%d/%d devices are supported" % (supported, len(devlist)))
-    return supported > 0
-
-
-@contextlib.contextmanager
-def defer_cleanup():
-    "Hold every deallocation off until the (outermost) block exits."
-    with current_context().defer_cleanup():
-        yield
-
-
-profiling = require_context(driver.profiling)
-profile_start = require_context(driver.profile_start)
-profile_stop = require_context(driver.profile_stop)
+    print("\t%d/%d devices are supported" % (usable, len(found)))
+    return usable > 0
 
 
 def is_available():

@@ -644,16 +644,14 @@ class MemoryPointer:
 
     def __init__(self, context, pointer, size, owner=None, finalizer=None):
         if isinstance(pointer, (c_void_p, c_size_t)):
-            pointer = pointer.value or 0
-        self.context = context
-        self.device_pointer = int(pointer or 0)
-        self.size = size
-        self._cuda_memsize_ = size
-        self.is_managed = finalizer is not None
+            pointer = pointer.value
+        address = int(pointer or 0)
+        self.context, self._owner = context, owner
+        self.device_pointer = self.handle = address
+        self.size = self._cuda_memsize_ = size
         self.refct = 1
-        self.handle = self.device_pointer
-        self._owner = owner
-        if finalizer is not None:
+        self.is_managed = finalizer is not None
+        if self.is_managed:
             self._finalizer = weakref.finalize(self, finalizer)
 
     @property
@@ -758,32 +756,32 @@ class PinnedMemory(_HostBufferMixin):
 
 class OwnedPointer:
     """A counted reference to a MemoryPointer, optionally looking at a sub-range
-    of it (reference :1848-1880)."""
+    of it (reference :1848-1880).  Creating one bumps the owner's `refct`; when it
+    is collected the count drops again and the owner is freed at zero.  Attribute
+    access falls through to the pointer it looks at."""
 
     def __init__(self, memptr, view=None):
-        self._mem = memptr
-        if view is None:
-            self._view = self._mem
-        else:
+        target = memptr if view is None else view
+        if view is not None:
             assert not view.is_managed
-            self._view = view
-        mem = self._mem
-
-        def deref():
-            try:
-                mem.refct -= 1
-                assert mem.refct >= 0
-                if mem.refct == 0:
-                    mem.free()
-            except ReferenceError:
-                pass
-
-        self._mem.refct += 1
-        weakref.finalize(self, deref)
-        self.device_ctypes_pointer = self._view.device_ctypes_pointer
+        self._mem, self._view = memptr, target
+        # used on every kernel argument: worth a real attribute
+        self.device_ctypes_pointer = target.device_ctypes_pointer
+        memptr.refct += 1
+        weakref.finalize(self, _drop_reference, memptr)
 
     def __getattr__(self, fname):
         return getattr(self._view, fname)
+
+
+def _drop_reference(mem):
+    try:
+        mem.refct -= 1
+        assert mem.refct >= 0
+        if mem.refct == 0:
+            mem.free()
+    except ReferenceError:
+        pass      # the owner went first; nothing left to release
 
 
 class MappedOwnedPointer(OwnedPointer, _HostBufferMixin):
