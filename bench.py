@@ -1,14 +1,14 @@
 #!/usr/bin/env python
 """Benchmark of the hot path on one MI355X.
 
-Default workload (BASELINE.json configs[1], the configuration the metric is quoted
+Default workload (the configuration the headline metric is quoted
 on): cuda.reduce float32 sum over 2^28 elements N(0,1), seed 1.  A "step" is one
 full reduction, issued through the public API into a device result slot; inputs
 are resident in HBM before the clock starts.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
-Other workloads (--workload) report the same line for the remaining BASELINE
+Other workloads (--workload) report the same line for the remaining benchmark
 configurations: reduce_f32_max, reduce_f64_sum, reduce_i64_sum, transpose_f32,
 transpose_f64, transpose_i16, rng_init, rng_uniform_f32, rng_normal_f64,
 batched_reduce, copy_f32 (counter calibration).

@@ -137,10 +137,10 @@ def test_montecarlo_integration_end_to_end():
         assert abs(est - want) < 1e-3
 
 
-# ---- BASELINE config 4, full size -----------------------------------------------------
+# ---- full-size case: 2^24 generators -----------------------------------------------------
 
 @pytest.mark.parametrize("start", [0, 5])
-def test_config4_states_2_pow_24(start):
+def test_fullsize_states_2_pow_24(start):
     n = 2**24
     states = cuda.random.create_xoroshiro128p_states(n, seed=42, subsequence_start=start)
     got = states.copy_to_host()
@@ -149,7 +149,7 @@ def test_config4_states_2_pow_24(start):
     assert got.tobytes() == want.tobytes()
 
 
-def test_config4_uniform_float32_2_pow_30_and_normal_float64():
+def test_fullsize_uniform_float32_2_pow_30_and_normal_float64():
     n, count = 2**24, 64
     host_states = cref.init_states(n, 42, 0)
     states = cuda.to_device(host_states)

@@ -120,7 +120,7 @@ def test_runs_are_bitwise_reproducible():
 
 
 def test_stream_and_result_slot_round_robin():
-    """BASELINE config 5 in small: independent row sums issued over 4 streams into
+    """The batched-reduction case in small: independent row sums issued over 4 streams into
     slots of one device vector."""
     rng = np.random.default_rng(3)
     rows, cols = 64, 65536
@@ -141,9 +141,9 @@ def test_stream_and_result_slot_round_robin():
     assert v.tobytes() == got[5].tobytes()
 
 
-# ---- BASELINE config 2: full HBM-scale inputs, seed 1 --------------------------------
+# ---- full HBM-scale inputs, seed 1 ---------------- --------------------------------
 
-def test_config2_float32_sum_and_max_2_pow_28():
+def test_fullsize_float32_sum_and_max_2_pow_28():
     n = 2**28
     _say("generating f32", n)
     a = np.random.default_rng(1).standard_normal(n, dtype=np.float32)
@@ -159,7 +159,7 @@ def test_config2_float32_sum_and_max_2_pow_28():
     assert mx == a.max() == cref.tree("max", a, -np.inf)
 
 
-def test_config2_float64_sum_2_pow_27():
+def test_fullsize_float64_sum_2_pow_27():
     n = 2**27
     a = np.random.default_rng(1).standard_normal(n)
     got = sum_reduce(cuda.to_device(a))
@@ -169,7 +169,7 @@ def test_config2_float64_sum_2_pow_27():
     assert abs(float(got) - float(cref.tree("add", a))) <= 2 * tol
 
 
-def test_config2_int64_sum_2_pow_28_bit_exact():
+def test_fullsize_int64_sum_2_pow_28_bit_exact():
     n = 2**28
     a = np.random.default_rng(1).integers(-2**20, 2**20, n, dtype=np.int64, endpoint=True)
     got = sum_reduce(cuda.to_device(a))

@@ -117,9 +117,9 @@ def test_row_padded_inputs_and_outputs():
     np.testing.assert_array_equal(dst_full.copy_to_host(), want)
 
 
-# ---- BASELINE config 3, full size, seed 2 ------------------------------------------------
+# ---- full-size matrices, seed 2 --------- ------------------------------------------------
 
-def test_config3_float32_16384_square():
+def test_fullsize_float32_16384_square():
     a = np.random.default_rng(2).random((16384, 16384), dtype=np.float32)
     d = cuda.to_device(a)
     t = d.T
@@ -129,14 +129,14 @@ def test_config3_float32_16384_square():
     assert _same_bytes(back, a)
 
 
-def test_config3_float64_ragged_12345_by_6789():
+def test_fullsize_float64_ragged_12345_by_6789():
     a = np.random.default_rng(2).random((12345, 6789))
     got = cuda.to_device(a).T.copy_to_host()
     assert got.shape == (6789, 12345)
     assert _same_bytes(got, a.T)
 
 
-def test_config3_int16_8192_by_32768():
+def test_fullsize_int16_8192_by_32768():
     a = np.random.default_rng(2).integers(-32768, 32767, (8192, 32768), dtype=np.int16, endpoint=True)
     got = cuda.to_device(a).T.copy_to_host()
     assert _same_bytes(got, a.T)

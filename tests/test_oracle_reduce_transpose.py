@@ -150,7 +150,7 @@ def test_minmax_follow_python_semantics_for_nan_and_signed_zero():
 
 def test_fold_matches_simulator_path():
     rng = np.random.default_rng(0)
-    a = rng.uniform(-1, 1, 65536).astype(np.float32)       # BASELINE config 1 input
+    a = rng.uniform(-1, 1, 65536).astype(np.float32)       # the 65536-element simulator case
     got = sim.Reduce(lambda x, y: x + y)(a[:4096], init=0)
     assert isinstance(got, np.float32)
     assert got == cref.fold("add", a[:4096], 0)
