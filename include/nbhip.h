@@ -130,13 +130,15 @@ size_t nbh_reduce_scratch_bytes(void);
 /* kernels/reduction.py:194-265 Reduce.__call__ together with the kernels it
  * launches (:15-166).  Computes
  *     out[0] = init (op) in[0] (op) in[1] (op) ... (op) in[n-1]
- * for n >= 1 contiguous elements of `dtype` in device memory, in one launch and
- * fully asynchronously on `stream`.  `init` points to one element of `dtype` in
- * HOST memory (read before the call returns); `out` is one element in DEVICE
- * memory (what `res[:1]` is in the reference).  The association order differs
- * from the reference's (integer results are identical; floating-point sums agree
- * within rounding, |err| <= 2 n eps sum|x|), and is the same on every run. */
-int nbh_reduce(int op, int dtype, const void *in, int64_t n, const void *init, void *out,
+ * for n >= 1 elements of `dtype` in device memory, `in_stride` bytes apart (a
+ * multiple of the element size, any sign; the element size itself selects the
+ * 128-bit streaming path), in one launch and fully asynchronously on `stream`.
+ * `init` points to one element of `dtype` in HOST memory (read before the call
+ * returns); `out` is one element in DEVICE memory (what `res[:1]` is in the
+ * reference).  The association order differs from the reference's (integer
+ * results are identical; floating-point sums agree within rounding,
+ * |err| <= 2 n eps sum|x|), and is the same on every run. */
+int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                void *scratch, size_t scratch_bytes, nbh_stream_t stream);
 
 /* ---- transpose ------------------------------------------------------------ */

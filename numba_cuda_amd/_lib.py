@@ -56,7 +56,7 @@ SIGNATURES = {
     "nbh_stream_wait_event": (c_int, [c_vp, c_vp]),
     "nbh_event_elapsed_ms": (c_int, [P(ctypes.c_float), c_vp, c_vp]),
     "nbh_reduce_scratch_bytes": (c_size, []),
-    "nbh_reduce": (c_int, [c_int, c_int, c_vp, c_i64, c_vp, c_vp, c_vp, c_size, c_vp]),
+    "nbh_reduce": (c_int, [c_int, c_int, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_size, c_vp]),
     "nbh_transpose": (c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "nbh_assign": (c_int, [c_vp, c_vp, c_int, P(c_i64), P(c_i64), P(c_i64), c_i64, c_vp]),
     "nbh_xoro_init_states": (c_int, [c_vp, c_i64, c_u64, c_u64, c_vp]),

@@ -145,9 +145,12 @@ template <typename A> struct BitsOf {
 };
 
 // ---- the kernel ------------------------------------------------------------------
-template <typename T, typename Op>
+// STRIDED: the items are `stride` bytes apart (any sign) instead of packed; they are
+// then read one by one, `nvec` counts items and `head` is 0.
+template <typename T, typename Op, bool STRIDED>
 __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in, int64_t n, int64_t head,
-                                                        int64_t nvec, T init, T *__restrict__ out,
+                                                        int64_t nvec, int64_t stride, T init,
+                                                        T *__restrict__ out,
                                                         uint64_t *__restrict__ partials_raw,
                                                         unsigned *__restrict__ ticket)
 {
@@ -174,31 +177,46 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
         end = nvec;
 
     int64_t i = begin + tid;
-    for (; i + (kUnroll - 1) * kBlock < end; i += kUnroll * kBlock) {
-        VecT v[kUnroll];
+    if constexpr (STRIDED) {
+        const char *__restrict__ bytes = reinterpret_cast<const char *>(in);
+        for (; i + (kUnroll - 1) * kBlock < end; i += kUnroll * kBlock) {
+            T v[kUnroll];
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-            v[u] = __builtin_nontemporal_load(&vin[i + u * kBlock]);
+            for (int u = 0; u < kUnroll; ++u)
+                v[u] = *reinterpret_cast<const T *>(bytes + (i + u * kBlock) * stride);
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+            for (int u = 0; u < kUnroll; ++u)
+                acc[u % V] = Op::apply(acc[u % V], (A)v[u]);
+        }
+        for (; i < end; i += kBlock)
+            acc[0] = Op::apply(acc[0], (A) * reinterpret_cast<const T *>(bytes + i * stride));
+    } else {
+        for (; i + (kUnroll - 1) * kBlock < end; i += kUnroll * kBlock) {
+            VecT v[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+                v[u] = __builtin_nontemporal_load(&vin[i + u * kBlock]);
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    acc[j] = Op::apply(acc[j], (A)v[u][j]);
+        }
+        for (; i < end; i += kBlock) {
+            VecT v = __builtin_nontemporal_load(&vin[i]);
 #pragma unroll
             for (int j = 0; j < V; ++j)
-                acc[j] = Op::apply(acc[j], (A)v[u][j]);
-    }
-    for (; i < end; i += kBlock) {
-        VecT v = __builtin_nontemporal_load(&vin[i]);
-#pragma unroll
-        for (int j = 0; j < V; ++j)
-            acc[j] = Op::apply(acc[j], (A)v[j]);
-    }
+                acc[j] = Op::apply(acc[j], (A)v[j]);
+        }
 
-    // elements outside the aligned body: fewer than 2 V, one per lane of workgroup 0
-    if (blockIdx.x == 0) {
-        const int64_t tail_begin = head + nvec * V;
-        if (tid < head)
-            acc[0] = Op::apply(acc[0], (A)in[tid]);
-        else if (tail_begin + (tid - head) < n)
-            acc[0] = Op::apply(acc[0], (A)in[tail_begin + (tid - head)]);
+        // elements outside the aligned body: fewer than 2 V, one per lane of workgroup 0
+        if (blockIdx.x == 0) {
+            const int64_t tail_begin = head + nvec * V;
+            if (tid < head)
+                acc[0] = Op::apply(acc[0], (A)in[tid]);
+            else if (tail_begin + (tid - head) < n)
+                acc[0] = Op::apply(acc[0], (A)in[tail_begin + (tid - head)]);
+        }
     }
 
     A mine = acc[0];
@@ -242,19 +260,24 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
 }
 
 template <typename T, typename Op>
-int launch(const void *in, int64_t n, const void *init, void *out, void *scratch, hipStream_t stream)
+int launch(const void *in, int64_t n, int64_t stride, const void *init, void *out, void *scratch,
+           hipStream_t stream)
 {
     constexpr int V = 16 / (int)sizeof(T);
     const uintptr_t addr = (uintptr_t)in;
-    if (addr % sizeof(T) != 0 || ((uintptr_t)out) % sizeof(T) != 0)
+    if (addr % sizeof(T) != 0 || ((uintptr_t)out) % sizeof(T) != 0 || stride % (int64_t)sizeof(T) != 0)
         return (int)hipErrorInvalidValue;
-    int64_t head = (int64_t)(((16 - (addr % 16)) % 16) / sizeof(T));
-    if (head > n)
-        head = n;
-    const int64_t nvec = (n - head) / V;
+    const bool strided = stride != (int64_t)sizeof(T) && n > 1;
+    int64_t head = 0, units = n;  // units: vectors when packed, items when strided
+    if (!strided) {
+        head = (int64_t)(((16 - (addr % 16)) % 16) / sizeof(T));
+        if (head > n)
+            head = n;
+        units = (n - head) / V;
+    }
 
     const int64_t per_block = (int64_t)kBlock * kUnroll;
-    int64_t grid = (nvec + per_block - 1) / per_block;
+    int64_t grid = (units + per_block - 1) / per_block;
     int64_t cap = (int64_t)nbh_cu_count() * kGridPerCU;
     if (cap > kMaxGrid)
         cap = kMaxGrid;
@@ -267,19 +290,24 @@ int launch(const void *in, int64_t n, const void *init, void *out, void *scratch
     __builtin_memcpy(&init_value, init, sizeof(T));
     unsigned *ticket = reinterpret_cast<unsigned *>(scratch);
     uint64_t *partials = reinterpret_cast<uint64_t *>((char *)scratch + kHeaderBytes);
-    hipLaunchKernelGGL((reduce_kernel<T, Op>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
-                       (const T *)in, n, head, nvec, init_value, (T *)out, partials, ticket);
+    if (strided)
+        hipLaunchKernelGGL((reduce_kernel<T, Op, true>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
+                           (const T *)in, n, head, units, stride, init_value, (T *)out, partials, ticket);
+    else
+        hipLaunchKernelGGL((reduce_kernel<T, Op, false>), dim3((unsigned)grid), dim3(kBlock), 0, stream,
+                           (const T *)in, n, head, units, stride, init_value, (T *)out, partials, ticket);
     return nbh_launch_status();
 }
 
 template <typename T>
-int launch_op(int op, const void *in, int64_t n, const void *init, void *out, void *scratch, hipStream_t s)
+int launch_op(int op, const void *in, int64_t n, int64_t stride, const void *init, void *out, void *scratch,
+              hipStream_t s)
 {
     switch (op) {
-    case NBH_ADD: return launch<T, OpAdd>(in, n, init, out, scratch, s);
-    case NBH_MUL: return launch<T, OpMul>(in, n, init, out, scratch, s);
-    case NBH_MAX: return launch<T, OpMax>(in, n, init, out, scratch, s);
-    case NBH_MIN: return launch<T, OpMin>(in, n, init, out, scratch, s);
+    case NBH_ADD: return launch<T, OpAdd>(in, n, stride, init, out, scratch, s);
+    case NBH_MUL: return launch<T, OpMul>(in, n, stride, init, out, scratch, s);
+    case NBH_MAX: return launch<T, OpMax>(in, n, stride, init, out, scratch, s);
+    case NBH_MIN: return launch<T, OpMin>(in, n, stride, init, out, scratch, s);
     default: return (int)hipErrorInvalidValue;
     }
 }
@@ -290,24 +318,24 @@ extern "C" {
 
 size_t nbh_reduce_scratch_bytes(void) { return kScratchBytes; }
 
-int nbh_reduce(int op, int dtype, const void *in, int64_t n, const void *init, void *out, void *scratch,
-               size_t scratch_bytes, nbh_stream_t stream)
+int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
+               void *scratch, size_t scratch_bytes, nbh_stream_t stream)
 {
     if (!in || !init || !out || !scratch || n < 1 || scratch_bytes < kScratchBytes ||
         ((uintptr_t)scratch) % 8 != 0)
         return (int)hipErrorInvalidValue;
     hipStream_t s = nbh_hip_stream(stream);
     switch (dtype) {
-    case NBH_I8: return launch_op<int8_t>(op, in, n, init, out, scratch, s);
-    case NBH_I16: return launch_op<int16_t>(op, in, n, init, out, scratch, s);
-    case NBH_I32: return launch_op<int32_t>(op, in, n, init, out, scratch, s);
-    case NBH_I64: return launch_op<int64_t>(op, in, n, init, out, scratch, s);
-    case NBH_U8: return launch_op<uint8_t>(op, in, n, init, out, scratch, s);
-    case NBH_U16: return launch_op<uint16_t>(op, in, n, init, out, scratch, s);
-    case NBH_U32: return launch_op<uint32_t>(op, in, n, init, out, scratch, s);
-    case NBH_U64: return launch_op<uint64_t>(op, in, n, init, out, scratch, s);
-    case NBH_F32: return launch_op<float>(op, in, n, init, out, scratch, s);
-    case NBH_F64: return launch_op<double>(op, in, n, init, out, scratch, s);
+    case NBH_I8: return launch_op<int8_t>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_I16: return launch_op<int16_t>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_I32: return launch_op<int32_t>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_I64: return launch_op<int64_t>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_U8: return launch_op<uint8_t>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_U16: return launch_op<uint16_t>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_U32: return launch_op<uint32_t>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_U64: return launch_op<uint64_t>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_F32: return launch_op<float>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_F64: return launch_op<double>(op, in, n, in_stride, init, out, scratch, s);
     default: return (int)hipErrorInvalidValue;
     }
 }

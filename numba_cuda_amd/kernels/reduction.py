@@ -186,8 +186,6 @@ class Reduce:
         if not _driver.is_device_memory(arr):
             # host input: implicit transfer, as a kernel argument would get
             arr, _ = devicearray.auto_device(arr, stream=stream)
-        if arr.strides[0] != dtype.itemsize:
-            raise NotImplementedError("Reduce needs a unit-stride array; got strides %s" % (arr.strides,))
 
         hstream = stream.handle if type(stream) is _driver.Stream else _driver._stream_handle(stream)
         scratch_ptr, slot, scratch_bytes = ctx.reduce_scratch(hstream)
@@ -199,7 +197,8 @@ class Reduce:
             out_ptr = slot      # per-stream result slot: no allocation per call
         init_ptr = _init_buffer(dtype, init)
         drv = _driver.driver
-        rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size, init_ptr,
+        rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size,
+                                arr.strides[0], init_ptr,
                                 out_ptr, scratch_ptr, scratch_bytes, hstream or None)
         if rc:
             drv.check("nbh_reduce", rc)

@@ -199,3 +199,23 @@ def test_back_to_back_reductions_never_see_stale_partials():
     want = csum[offs + sizes] - csum[offs] + np.arange(calls)
     bad = np.nonzero(got != want)[0]
     assert bad.size == 0, (bad[:10], got[bad[:10]], want[bad[:10]])
+
+
+def test_strided_and_reversed_views():
+    """The reference indexes `arr[i]`, so any 1-D view reduces; here non-unit strides
+    take the item-by-item path of the same kernel."""
+    rng = np.random.default_rng(21)
+    a = rng.integers(-10**6, 10**6, 200_003).astype(np.int64)
+    d = cuda.to_device(a)
+    mx = cuda.Reduce(lambda x, y: max(x, y))
+    for view, want in ((d[::2], a[::2]), (d[1::3], a[1::3]), (d[::-1], a[::-1]), (d[5000:100:-7], a[5000:100:-7]),
+                       (d[::1000], a[::1000]), (d[7:8:5], a[7:8:5])):
+        assert sum_reduce(view, init=3) == want.sum() + 3
+        assert mx(view, init=-10**9) == want.max()
+    m = rng.standard_normal((300, 257)).astype(np.float32)
+    dm = cuda.to_device(m)
+    col = dm[:, 5]                                   # a column: stride = one row
+    exact, sum_abs = cref.sum_exact(np.ascontiguousarray(m[:, 5]))
+    assert abs(float(sum_reduce(col)) - exact) <= 2 * 300 * np.finfo(np.float32).eps * sum_abs
+    b = rng.integers(-128, 127, 70_001).astype(np.int8)
+    assert sum_reduce(cuda.to_device(b)[::3]) == cref.fold("add", np.ascontiguousarray(b[::3]))

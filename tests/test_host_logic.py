@@ -47,7 +47,7 @@ def test_library_loads_without_a_gpu_and_reports_errors_by_name():
     n = ctypes.c_int(-1)
     assert lib.nbh_device_count(ctypes.byref(n)) == 0 and n.value >= 0
     # argument checking happens before any device work
-    assert lib.nbh_reduce(0, 99, None, 1, None, None, None, 0, None) != 0
+    assert lib.nbh_reduce(0, 99, None, 1, 4, None, None, None, 0, None) != 0
     assert lib.nbh_transpose(None, None, -1, 1, 4, 4, 4, 4, 4, None) != 0
     assert lib.nbh_transpose(None, None, 0, 5, 4, 4, 4, 4, 4, None) == 0      # empty: nothing to do
 
