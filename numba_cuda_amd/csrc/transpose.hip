@@ -136,6 +136,124 @@ __global__ __launch_bounds__(64 * ShapeOf<E>::WR * ShapeOf<E>::WC) void transpos
     }
 }
 
+// Output rows that do not start on a 128-byte line.  With the packet kernel every
+// 128-byte piece a wavefront stores would straddle two lines (measured: float32,
+// 16388 rows, 4.1 TB/s against 5.4 TB/s when only the INPUT rows straddle).  Here a
+// workgroup walks down a strip of the input, TR rows at a time, through a ring of
+// RING = TR + L rows in LDS (L = items per line), and for every output row c it
+// writes the items r in [lo(c), hi(c)), both ends rounded down to the nearest r at
+// which output row c crosses a line boundary: every store covers whole lines.  What
+// lies below hi(c) stays in the ring for the next step, so nothing is read twice
+// except the L rows above the start of a strip.
+template <int E> struct ShearOf;   // RING must be a power of two
+template <> struct ShearOf<1> { static constexpr int RING = 512, TC = 64; };
+template <> struct ShearOf<2> { static constexpr int RING = 256, TC = 64; };
+template <> struct ShearOf<4> { static constexpr int RING = 128, TC = 32; };
+template <> struct ShearOf<8> { static constexpr int RING = 64, TC = 32; };
+template <> struct ShearOf<16> { static constexpr int RING = 32, TC = 32; };
+constexpr int kStripSteps = 8;  // steps of TR rows per workgroup
+
+template <int E>
+__global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__restrict__ in, char *__restrict__ out,
+                                                               int64_t rows, int64_t cols, int64_t in_s0,
+                                                               int64_t out_s0, int64_t strips_r)
+{
+    using Item = typename ItemOf<E>::type;
+    constexpr int V = 16 / E;    // items per packet
+    constexpr int L = 128 / E;   // items per cache line
+    constexpr int RING = ShearOf<E>::RING, TC = ShearOf<E>::TC;
+    constexpr int TR = RING - L;
+    constexpr int PPR = TC / V;  // packets per tile row
+    __shared__ Item ring[RING][TC + 1];
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int64_t tile_c = (int64_t)blockIdx.x / strips_r;
+    const int64_t strip = (int64_t)blockIdx.x % strips_r;
+    const int64_t C0 = tile_c * TC;
+    const int64_t strip_begin = strip * (int64_t)(kStripSteps * TR);
+    int64_t strip_end = strip_begin + (int64_t)kStripSteps * TR;
+    const bool last_strip = strip == strips_r - 1;
+    if (last_strip)
+        strip_end = rows;
+
+    // A step's rows travel global -> registers -> ring, so that the loads of the next
+    // step are already in flight while this step's rows are being written out.
+    constexpr int NP = (RING * PPR + kThreads - 1) / kThreads;  // packets per thread, at most
+    union Pack {
+        u32x4 pk;
+        Item it[V];
+    };
+    Pack held[NP];
+
+    auto fetch = [&](int64_t from, int64_t to) {  // rows [from, to) -> held
+        const int count = (int)(to - from) * PPR;
+#pragma unroll
+        for (int k = 0; k < NP; ++k) {
+            const int idx = tid + k * kThreads;
+            if (idx >= count)
+                break;
+            const int64_t gr = from + idx / PPR;
+            const int64_t gc = C0 + (int64_t)(idx % PPR) * V;
+            if (gr < 0 || gc >= cols)
+                continue;
+            const char *src = in + gr * in_s0 + gc * E;
+            if (gc + V <= cols) {
+                held[k].pk = reinterpret_cast<const Packet<E> *>(src)->v;
+            } else {
+                for (int j = 0; j < V; ++j)
+                    if (gc + j < cols)
+                        held[k].it[j] = *reinterpret_cast<const Item *>(src + (int64_t)j * E);
+            }
+        }
+    };
+    auto park = [&](int64_t from, int64_t to) {  // held -> ring (columns beyond the edge carry junk, never stored)
+        const int count = (int)(to - from) * PPR;
+#pragma unroll
+        for (int k = 0; k < NP; ++k) {
+            const int idx = tid + k * kThreads;
+            if (idx >= count)
+                break;
+            const int64_t gr = from + idx / PPR;
+            if (gr < 0)
+                continue;
+            Item *dst = &ring[gr & (RING - 1)][(idx % PPR) * V];
+#pragma unroll
+            for (int j = 0; j < V; ++j)
+                dst[j] = held[k].it[j];
+        }
+    };
+
+    fetch(strip_begin - L, strip_begin);  // what the first step needs from above
+    park(strip_begin - L, strip_begin);
+    int64_t R0 = strip_begin;
+    int64_t step_end = (R0 + TR < strip_end) ? R0 + TR : strip_end;
+    fetch(R0, step_end);
+    while (R0 < strip_end) {
+        park(R0, step_end);
+        __syncthreads();
+        const int64_t next = step_end;
+        const int64_t next_end = (next + TR < strip_end) ? next + TR : strip_end;
+        if (next < strip_end)
+            fetch(next, next_end);
+        for (int lc = wave; lc < TC; lc += kThreads / 64) {
+            const int64_t c = C0 + lc;
+            if (c >= cols)
+                break;
+            char *row = out + c * out_s0;
+            const int64_t phase = (int64_t)(((uintptr_t)row % 128) / E);  // line offset of item 0, in items
+            int64_t lo = R0 - (phase + R0) % L;
+            if (lo < 0)
+                lo = 0;
+            const int64_t hi = (step_end == rows) ? rows : step_end - (phase + step_end) % L;
+            for (int64_t r = lo + lane; r < hi; r += 64)
+                *reinterpret_cast<Item *>(row + r * E) = ring[r & (RING - 1)][lc];
+        }
+        __syncthreads();  // the next step overwrites rows that were just read
+        R0 = next;
+        step_end = next_end;
+    }
+}
+
 // One lane per G-byte chunk of one item; chunk index fastest, then the output's
 // inner index, then its outer index.
 template <int G>
@@ -179,6 +297,21 @@ int launch_packets(const void *in, void *out, int64_t rows, int64_t cols, int64_
     return nbh_launch_status();
 }
 
+template <int E>
+int launch_sheared(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
+                   hipStream_t stream)
+{
+    constexpr int TR = ShearOf<E>::RING - 128 / E;
+    const int64_t strips_r = (rows + (int64_t)kStripSteps * TR - 1) / ((int64_t)kStripSteps * TR);
+    const int64_t tiles_c = (cols + ShearOf<E>::TC - 1) / ShearOf<E>::TC;
+    const int64_t blocks = strips_r * tiles_c;
+    if (blocks > 0x7fffffffLL)
+        return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((transpose_sheared<E>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, (const char *)in,
+                       (char *)out, rows, cols, in_s0, out_s0, strips_r);
+    return nbh_launch_status();
+}
+
 template <int G>
 int launch_strided(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t in_s1,
                    int64_t out_s0, int64_t out_s1, int64_t itemsize, hipStream_t stream)
@@ -217,6 +350,18 @@ extern "C" int nbh_transpose(const void *in, void *out, int64_t rows, int64_t co
 
     const bool unit_inner = in_s1 == itemsize && out_s1 == itemsize && in_s0 > 0 && out_s0 > 0;
     if (unit_inner && g == itemsize) {  // item size is a power of two <= 16 and items are aligned
+        // output rows off the 128-byte grid and long enough for the shear to pay
+        const bool ragged_out = (((uint64_t)(uintptr_t)out | (uint64_t)out_s0) % 128) != 0 && rows * itemsize >= 512;
+        if (ragged_out) {
+            switch (itemsize) {
+            case 1: return launch_sheared<1>(in, out, rows, cols, in_s0, out_s0, s);
+            case 2: return launch_sheared<2>(in, out, rows, cols, in_s0, out_s0, s);
+            case 4: return launch_sheared<4>(in, out, rows, cols, in_s0, out_s0, s);
+            case 8: return launch_sheared<8>(in, out, rows, cols, in_s0, out_s0, s);
+            case 16: return launch_sheared<16>(in, out, rows, cols, in_s0, out_s0, s);
+            default: break;
+            }
+        }
         switch (itemsize) {
         case 1: return launch_packets<1>(in, out, rows, cols, in_s0, out_s0, s);
         case 2: return launch_packets<2>(in, out, rows, cols, in_s0, out_s0, s);

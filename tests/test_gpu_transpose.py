@@ -92,7 +92,7 @@ def test_T_and_transpose_api():
 @pytest.mark.parametrize("dtype", [np.int8, np.uint16, np.float32, np.int64, np.complex128,
                                    np.dtype("S3"), np.dtype("S12"), recordwith2darray])
 @pytest.mark.parametrize("shape", [(1, 1), (1, 300), (300, 1), (64, 64), (65, 63), (127, 129),
-                                   (257, 515), (1000, 777), (2049, 33)])
+                                   (257, 515), (1000, 777), (2049, 33), (7001, 131)])
 def test_every_item_size_and_ragged_shapes(shape, dtype):
     dtype = np.dtype(dtype)
     _say("transpose", shape, dtype)
