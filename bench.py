@@ -39,6 +39,8 @@ MEASURED_TRAFFIC = {
     "transpose_f32": 2148293558,
     # profiles/xoroshiro_fill_and_init_2p24.txt: 268 534 300 B fetched + 4 563 402 098 B written
     "rng_uniform_f32": 4831936398,
+    # profiles/transpose_sheared_f64_12345x6789.txt: 1 026 969 245 B fetched + 670 744 593 B written
+    "transpose_f64": 1697713838,
 }
 
 
@@ -129,7 +131,9 @@ def _workload(name, cuda):
 
         return dict(desc="transpose %s %dx%d, seed 2" % (host.dtype.name, host.shape[0], host.shape[1]),
                     dtype=host.dtype.name, algo_bytes=2 * host.nbytes, units=host.size, step=step,
-                    stream=stream, host=None, kernel="transpose_tiled", keep=(src, dst))
+                    stream=stream, host=None, keep=(src, dst),
+                    kernel={"transpose_f32": "transpose_packets<4, true>", "transpose_f64": "transpose_sheared<8>",
+                            "transpose_i16": "transpose_packets<2, true>"}[name])
     if name.startswith("rng_"):
         n = 2**24
         states = cuda.device_array(n, dtype=nrandom.xoroshiro128p_dtype)
