@@ -76,6 +76,10 @@ int nbh_device_synchronize(void);
  * cuMemFree its finalizer queues (:1316-1325) */
 int nbh_malloc(void **dptr, size_t nbytes);
 int nbh_free(void *dptr);
+/* cudadrv/driver.py:819-838 memallocmanaged (cuMemAllocManaged): memory addressable
+ * from the host and the device at the same address; attach_global != 0 ->
+ * attached to every stream, 0 -> host-attached.  Release with nbh_free. */
+int nbh_malloc_managed(void **ptr, size_t nbytes, int attach_global);
 /* cudadrv/driver.py:747-779 memhostalloc (cuMemHostAlloc / cuMemFreeHost).
  * flags: bit 0 portable, bit 1 device-mapped, bit 2 write-combined */
 int nbh_host_alloc(void **hptr, size_t nbytes, unsigned flags);

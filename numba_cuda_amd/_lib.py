@@ -33,6 +33,7 @@ SIGNATURES = {
     "nbh_device_synchronize": (c_int, []),
     "nbh_malloc": (c_int, [P(c_vp), c_size]),
     "nbh_free": (c_int, [c_vp]),
+    "nbh_malloc_managed": (c_int, [P(c_vp), c_size, c_int]),
     "nbh_host_alloc": (c_int, [P(c_vp), c_size, ctypes.c_uint]),
     "nbh_host_free": (c_int, [c_vp]),
     "nbh_host_register": (c_int, [c_vp, c_size, ctypes.c_uint]),

@@ -112,6 +112,19 @@ def mapped_array_like(ary, stream=0, portable=False, wc=False):
                         portable=portable, wc=wc)
 
 
+def managed_array(shape, dtype=np.float64, strides=None, order="C", stream=0, attach_global=True):
+    """Host ndarray in managed memory: the same address is valid on the host and on
+    the device, and the array can be passed wherever a device array is.
+    `attach_global=False` attaches the memory to the host only."""
+    shape, strides, dtype = prepare_shape_strides_dtype(shape, strides, dtype, order)
+    nbytes = driver.memory_size_from_info(shape, strides, dtype.itemsize)
+    mem = _ctx().memallocmanaged(nbytes, attach_global=attach_global)
+    ary = np.ndarray(shape=shape, strides=strides, dtype=dtype, order=order, buffer=mem.as_buffer())
+    out = np.ndarray.view(ary, type=devicearray.ManagedNDArray)
+    out.device_setup(mem, stream=stream)
+    return out
+
+
 def from_cuda_array_interface(desc, owner=None, sync=True):
     """Wrap the memory described by a __cuda_array_interface__ dict in a
     DeviceNDArray without copying; `owner` is kept alive by the result.  If the

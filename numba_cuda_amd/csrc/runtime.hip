@@ -105,6 +105,12 @@ int nbh_malloc(void **dptr, size_t nbytes)
     return (int)hipMalloc(dptr, nbytes);
 }
 int nbh_free(void *dptr) { return (int)hipFree(dptr); }
+int nbh_malloc_managed(void **ptr, size_t nbytes, int attach_global)
+{
+    if (!ptr)
+        return (int)hipErrorInvalidValue;
+    return (int)hipMallocManaged(ptr, nbytes, attach_global ? hipMemAttachGlobal : hipMemAttachHost);
+}
 
 int nbh_host_alloc(void **hptr, size_t nbytes, unsigned flags)
 {

@@ -465,12 +465,43 @@ class DeviceNDArray(DeviceNDArrayBase):
     _do_setitem = setitem
 
 
-class MappedNDArray(DeviceNDArrayBase, np.ndarray):
-    """A host array in pinned memory that the device can address."""
+class _HostVisibleArray(DeviceNDArrayBase, np.ndarray):
+    """An ndarray whose buffer the device can address too.  It is created as a view of
+    a plain ndarray (so DeviceNDArrayBase.__init__ never runs) and told its memory
+    with device_setup(); NumPy views of it (slices, reshapes) find their own device
+    range from the parent's."""
+
+    gpu_data = None
+    stream = 0
 
     def device_setup(self, gpu_data, stream=0):
         self.gpu_data = gpu_data
         self.stream = stream
+
+    def __array_finalize__(self, parent):
+        data = getattr(parent, "gpu_data", None)
+        if data is None or not isinstance(parent, _HostVisibleArray):
+            return
+        start = self.__array_interface__["data"][0] - parent.__array_interface__["data"][0]
+        if 0 <= start <= data.size:
+            self.gpu_data = data.view(start) if start else data
+            self.stream = parent.stream
+
+    @property
+    def _dummy(self):
+        return dummyarray.Array.from_desc(0, self.shape, self.strides, self.dtype.itemsize)
+
+    @property
+    def alloc_size(self):
+        return _driver.memory_size_from_info(self.shape, self.strides, self.dtype.itemsize)
+
+
+class MappedNDArray(_HostVisibleArray):
+    """A host array in pinned memory that the device can address."""
+
+
+class ManagedNDArray(_HostVisibleArray):
+    """A host array in managed memory (reference :848-855)."""
 
 
 # ---- constructors from host objects ------------------------------------------------------

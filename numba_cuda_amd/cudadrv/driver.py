@@ -388,6 +388,18 @@ class HostOnlyCUDAMemoryManager(BaseCUDAMemoryManager):
             return mem.own()
         return PinnedMemory(ctx, pointer, size, owner=owner, finalizer=finalizer)
 
+    def memallocmanaged(self, size, attach_global):
+        def allocator():
+            p = c_void_p()
+            driver.nbh_malloc_managed(byref(p), size, 1 if attach_global else 0)
+            return p.value or 0
+
+        ptr = self._attempt_allocation(allocator)
+        finalizer = _alloc_finalizer(self, ptr, ptr, size)
+        mem = ManagedMemory(weakref.proxy(self.context), ptr, size, finalizer=finalizer)
+        self.allocations[ptr] = mem
+        return mem.own()
+
     def reset(self):
         self.allocations.clear()
         self.deallocations.clear()
@@ -492,6 +504,9 @@ class Context:
 
     def memhostalloc(self, bytesize, mapped=False, portable=False, wc=False):
         return self.memory_manager.memhostalloc(bytesize, mapped, portable, wc)
+
+    def memallocmanaged(self, bytesize, attach_global=True):
+        return self.memory_manager.memallocmanaged(bytesize, attach_global)
 
     def mempin(self, owner, pointer, size, mapped=False):
         if mapped and not self.device.CAN_MAP_HOST_MEMORY:
@@ -735,6 +750,23 @@ class MappedMemory(AutoFreePointer, _HostBufferMixin):
         return MappedOwnedPointer(weakref.proxy(self))
 
 
+class ManagedMemory(AutoFreePointer, _HostBufferMixin):
+    """Managed memory: one address, valid on the host and on the device
+    (reference :1813-1845)."""
+
+    __cuda_memory__ = True
+
+    def __init__(self, context, pointer, size, owner=None, finalizer=None):
+        self.owned = owner
+        super().__init__(context, int(pointer), size, finalizer=finalizer)
+        self.host_pointer = int(pointer)
+        self._bufptr_ = self.host_pointer
+        self._buflen_ = self.size
+
+    def own(self):
+        return ManagedOwnedPointer(weakref.proxy(self))
+
+
 class PinnedMemory(_HostBufferMixin):
     """Page-locked host memory (reference :1770-1808)."""
 
@@ -785,6 +817,10 @@ def _drop_reference(mem):
 
 
 class MappedOwnedPointer(OwnedPointer, _HostBufferMixin):
+    pass
+
+
+class ManagedOwnedPointer(OwnedPointer, _HostBufferMixin):
     pass
 
 

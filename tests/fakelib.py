@@ -98,6 +98,10 @@ class FakeLib:
         self._out(out, addr)
         return 0
 
+    def nbh_malloc_managed(self, out, nbytes, attach_global):
+        self._log("malloc_managed", nbytes, attach_global)
+        return self.nbh_malloc(out, nbytes)
+
     def nbh_free(self, ptr):
         addr = _addr(ptr)
         self._log("free", addr)

@@ -290,5 +290,33 @@ def implicit_copy_warning(cuda):
     assert sum(issubclass(x.category, NumbaPerformanceWarning) for x in w) == 1
 
 
-ALL = [roundtrip_and_attributes, constructors, slicing_views, copies_and_compatibility,
+def managed_memory(cuda):
+    """One buffer seen from both sides (tests/cudadrv/test_managed_alloc.py:75-124,
+    tests/cudadrv/test_cuda_memory.py:49-51)."""
+    ctx = cuda.current_context()
+    mem = ctx.memallocmanaged(1024)
+    assert drv.is_device_memory(mem) and mem.size == 1024
+    for attach_global in (True, False):
+        ary = cuda.managed_array(100, dtype=np.double, attach_global=attach_global)
+        assert isinstance(ary, np.ndarray) and cuda.is_cuda_array(ary)
+        ary.fill(123.456)
+        assert all(ary == 123.456)
+        # the device reads what the host wrote ...
+        if type(drv.driver.lib).__name__ != "FakeLib":      # the fake library has no kernels
+            assert cuda.reduce(lambda a, b: max(a, b))(ary, init=-1.0) == 123.456
+        # ... and the host reads what the device wrote, after a synchronisation
+        drv.device_memset(ary, 0, ary.nbytes)
+        cuda.synchronize()
+        assert all(ary == 0.0)
+        ary[:] = np.arange(100.0)
+        d = cuda.to_device(np.zeros(100))
+        d.copy_to_device(ary)                         # device-to-device from managed memory
+        np.testing.assert_array_equal(d.copy_to_host(), np.arange(100.0))
+    m2 = cuda.managed_array((4, 6), dtype=np.int32, order="F")
+    assert m2.flags["F_CONTIGUOUS"] and m2.strides == (4, 16)
+    del mem, ary, m2
+    gc.collect()
+
+
+ALL = [managed_memory, roundtrip_and_attributes, constructors, slicing_views, copies_and_compatibility,
        reshape_view_ravel_split, streams_events_pinned, deferred_deallocation, implicit_copy_warning]

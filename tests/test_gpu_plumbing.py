@@ -33,6 +33,19 @@ def test_mapped_array_is_device_addressable():
     assert got == np.arange(1000, dtype=np.float32).sum()
 
 
+def test_numpy_views_of_managed_and_mapped_arrays_are_device_arguments():
+    for make in (cuda.managed_array, cuda.mapped_array):
+        m = make((8, 1000), dtype=np.float64)
+        m[:] = np.arange(8000.0).reshape(8, 1000)
+        row = m[3]                                   # NumPy view: same class, own device range
+        assert type(row) is type(m)
+        assert row.device_ctypes_pointer.value == m.device_ctypes_pointer.value + 3 * 8000
+        assert cuda.reduce(lambda a, b: a + b)(row) == np.arange(3000.0, 4000.0).sum()
+        t = cuda.kernels.transpose.transpose(m[:, :500])
+        np.testing.assert_array_equal(t.copy_to_host(), np.asarray(m)[:, :500].T)
+        cuda.synchronize()
+
+
 def test_cuda_array_interface_with_torch_tensors():
     """Zero-copy import of a PyTorch-ROCm tensor, checked against torch itself."""
     torch = pytest.importorskip("torch")
