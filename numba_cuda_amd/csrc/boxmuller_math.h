@@ -1,0 +1,158 @@
+// The two transcendental steps of Box-Muller, specialised to the arguments the
+// generators produce, each within one unit in the last place of double:
+//
+//   bm_log_f32(u)  natural logarithm of a float32 in (0, 1] (any positive normal
+//                  float32 works), evaluated in double; u == 0 gives -infinity.
+//   bm_cos_2pi(x)  cosine of a double in [0, 6.2832], i.e. of 2*pi*u.
+//
+// The general-purpose library routines spend most of their time on cases that
+// cannot occur here (subnormals, huge arguments, Payne-Hanek reduction): on
+// MI355X they cost 650 us (log) and 460 us (cos) per 2^28 normals against 150 us for
+// the square root and 530 us for everything else including the stores.
+//
+// Both functions are plain C++ so that a host build can sweep them against a
+// long-double reference; BM_FN is the only thing that differs between the builds.
+#pragma once
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+
+#ifdef __HIPCC__
+#define BM_FN __host__ __device__ __forceinline__
+#else
+#define BM_FN inline
+#endif
+
+namespace bm {
+
+// ---- logarithm -------------------------------------------------------------------
+// u = 2^e * m with m in [sqrt(1/2), sqrt(2)).  The 2^23 mantissa patterns of m are cut
+// into 128 runs of 2^16; run j has a centre c_j (1.0 for the run that contains 1.0)
+// and the table holds q_j = RN(1 / c_j) and t_j = -log(q_j) as a double-double, so that
+//     log(m) = t_j + log1p(r),  r = m * q_j - 1  (|r| <= 2^-8)
+// holds exactly.  t_hi keeps 42 fractional bits: e * ln2_hi + t_hi is then exact.
+struct LogTable {
+    double q[128];
+    double t_hi[128];
+    double t_lo[128];
+};
+constexpr uint32_t kSqrtHalfBits = 0x3f3504f3u;  // float32 bits of sqrt(1/2)
+
+inline float bm_bits_to_float(uint32_t b)
+{
+    float f;
+    std::memcpy(&f, &b, 4);
+    return f;
+}
+
+// Host side: fill the table (long double carries 64 bits, the table needs ~100
+// between t_hi and t_lo, which the split provides: t_hi is exact by construction).
+inline void build_log_table(LogTable &t)
+{
+    for (int j = 0; j < 128; ++j) {
+        const uint32_t first = kSqrtHalfBits + ((uint32_t)j << 16), last = first + 0xffffu;
+        const double lo = (double)bm_bits_to_float(first), hi = (double)bm_bits_to_float(last);
+        const double c = (lo <= 1.0 && 1.0 <= hi) ? 1.0 : 0.5 * (lo + hi);
+        const double q = 1.0 / c;
+        const long double full = -logl((long double)q);
+        const double hi_part = (double)(std::floor((double)full * 0x1p42) * 0x1p-42);
+        t.q[j] = q;
+        t.t_hi[j] = hi_part;
+        t.t_lo[j] = (double)(full - (long double)hi_part);
+    }
+}
+
+BM_FN double log_positive_f32(float u, const LogTable *__restrict__ tab)
+{
+    uint32_t bits;
+#ifdef __HIP_DEVICE_COMPILE__
+    bits = __float_as_uint(u);
+#else
+    std::memcpy(&bits, &u, 4);
+#endif
+    const uint32_t ix = bits - kSqrtHalfBits;
+    const int e = (int32_t)ix >> 23;
+    const uint32_t j = (ix >> 16) & 127u;
+    const uint32_t mbits = (ix & 0x007fffffu) + kSqrtHalfBits;
+    float mf;
+#ifdef __HIP_DEVICE_COMPILE__
+    mf = __uint_as_float(mbits);
+#else
+    std::memcpy(&mf, &mbits, 4);
+#endif
+    const double m = (double)mf, fe = (double)e;
+    // r + r_lo = m * q_j - 1 exactly: where t_j is small, r is as large as the result
+    // and its own rounding would show
+    const double q = tab->q[j];
+    const double mq = m * q;
+    const double r_lo = __builtin_fma(m, q, -mq);
+    const double r = mq - 1.0;
+    // log1p(r) - r, |r| <= 2^-8: the r^8 / 8 term is below 2^-67
+    double p = __builtin_fma(r, 1.0 / 7.0, -1.0 / 6.0);
+    p = __builtin_fma(r, p, 1.0 / 5.0);
+    p = __builtin_fma(r, p, -1.0 / 4.0);
+    p = __builtin_fma(r, p, 1.0 / 3.0);
+    p = __builtin_fma(r, p, -0.5);
+    p = (r * r) * p;
+    p = __builtin_fma(-r, r_lo, p);                    // d/dr (log1p(r) - r) = -r to first order
+    const double ln2_hi = 0x1.62e42feep-1;             // 32 bits of ln 2
+    const double ln2_lo = 0x1.a39ef35793c76p-33;       // ln 2 - ln2_hi
+    const double hi = __builtin_fma(fe, ln2_hi, tab->t_hi[j]);  // exact
+    // s + err = hi + r exactly: hi is zero (run of 1.0, e = 0) or |hi| > |r|
+    const double s = hi + r;
+    const double err = r - (s - hi);
+    const double lo = ((__builtin_fma(fe, ln2_lo, tab->t_lo[j]) + r_lo) + p) + err;
+    return s + lo;
+}
+
+BM_FN double bm_log_f32(float u, const LogTable *__restrict__ tab)
+{
+    const double v = log_positive_f32(u, tab);
+    return (u == 0.0f) ? -HUGE_VAL : v;
+}
+
+// ---- cosine ------------------------------------------------------------------------
+// x = n * pi/2 + (y0 + y1), n = 0..4, |y0| <= pi/4 (+ a rounding's worth), with pi/2
+// carried to 119 bits in three pieces so that y0 + y1 is good to 2^-65 relative even
+// for x = RN(pi/2), where everything but 6e-17 cancels.  On [-pi/4, pi/4], with
+// z = y0^2 (coefficients S1..S6, C1..C6: the minimax sets of fdlibm's __kernel_sin /
+// __kernel_cos),
+//     sin(y0 + y1) = y0 + [ y0 z  (S1 + z (S2 + ... z S6)) + y1 (1 - z/2) ]
+//     cos(y0 + y1) = w  + [ z^2   (C1 + z (C2 + ... z C6)) + ((1 - w) - z/2) - y0 y1 ],  w = 1 - z/2
+// have the same shape, base + fma(factor, Horner(z), tail).  Double-precision
+// instructions are what bounds the generators, so the quadrant picks coefficients,
+// factor, tail and base per lane (32-bit selects) and ONE Horner chain runs.
+BM_FN double bm_cos_2pi(double x)
+{
+    const double inv_pio2 = 0x1.45f306dc9c883p-1;
+    const double pio2_1 = 0x1.921fb544p+0;             // first 33 bits of pi/2
+    const double pio2_2 = 0x1.0b4611a6p-34;            // next 33 bits
+    const double pio2_2t = 0x1.3198a2e037073p-69;      // pi/2 - pio2_1 - pio2_2
+    const double fn = __builtin_rint(x * inv_pio2);
+    const int n = (int)fn;
+    const double t = __builtin_fma(-fn, pio2_1, x);    // exact: fn * pio2_1 has 36 bits
+    const double w = fn * pio2_2;                      // exact
+    const double r = t - w;
+    const double w2 = __builtin_fma(fn, pio2_2t, -((t - r) - w));
+    const double y0 = r - w2;
+    const double y1 = (r - y0) - w2;
+
+    const bool odd = (n & 1) != 0;                     // odd quadrant: -+sin, even: +-cos
+    const double z = y0 * y0;
+    const double hz = 0.5 * z;
+    const double wc = 1.0 - hz;
+    double q = odd ? 0x1.5d93a5acfd57cp-33 : -0x1.8fae9be8838d4p-37;       // S6 : C6
+    q = __builtin_fma(z, q, odd ? -0x1.ae5e68a2b9cebp-26 : 0x1.1ee9ebdb4b1c4p-29);   // S5 : C5
+    q = __builtin_fma(z, q, odd ? 0x1.71de357b1fe7dp-19 : -0x1.27e4f809c52adp-22);   // S4 : C4
+    q = __builtin_fma(z, q, odd ? -0x1.a01a019c161d5p-13 : 0x1.a01a019cb159p-16);    // S3 : C3
+    q = __builtin_fma(z, q, odd ? 0x1.111111110f8a6p-7 : -0x1.6c16c16c15177p-10);    // S2 : C2
+    q = __builtin_fma(z, q, odd ? -0x1.5555555555549p-3 : 0x1.555555555554cp-5);     // S1 : C1
+    const double factor = z * (odd ? y0 : z);
+    const double tail = odd ? y1 * wc : __builtin_fma(-y0, y1, (1.0 - wc) - hz);
+    const double base = odd ? y0 : wc;
+    const double pick = base + __builtin_fma(factor, q, tail);
+    // cos(n*pi/2 + y): n&3 = 0: cos y, 1: -sin y, 2: -cos y, 3: sin y
+    return (((n + 1) & 2) != 0) ? -pick : pick;
+}
+
+}  // namespace bm

@@ -23,6 +23,8 @@
 //
 // HBM roofline: out bytes written + 2 * 16 bytes of state per generator.
 #include "common.h"
+#include "boxmuller_math.h"
+#include <type_traits>
 
 #include <mutex>
 
@@ -148,6 +150,34 @@ int device_table(const U128 **out)
             return (int)e;
         }
         cache[dev] = (const U128 *)d;
+    }
+    *out = cache[dev];
+    return 0;
+}
+
+// Device copy of the logarithm table of the normal generators (3 KiB), one per
+// device, made on first use and kept for the life of the process.
+int device_log_table(const bm::LogTable **out)
+{
+    constexpr int kMaxDev = 64;
+    static const bm::LogTable *cache[kMaxDev] = {};
+    static std::mutex mu;
+    int dev = 0;
+    NBH_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDev)
+        return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!cache[dev]) {
+        bm::LogTable host;
+        bm::build_log_table(host);
+        void *d = nullptr;
+        NBH_TRY(hipMalloc(&d, sizeof(bm::LogTable)));
+        hipError_t e = hipMemcpy(d, &host, sizeof(bm::LogTable), hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(d);
+            return (int)e;
+        }
+        cache[dev] = (const bm::LogTable *)d;
     }
     *out = cache[dev];
     return 0;
@@ -337,7 +367,7 @@ __device__ __forceinline__ double unit_double(uint64_t x)
 struct UniformF32 {
     using value_type = float;
     static constexpr bool kHeavy = false;
-    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1)
+    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1, const bm::LogTable * = nullptr)
     {
         // the exact value in double, then one rounding to float
         return (float)unit_double(next_d(s0, s1));
@@ -346,7 +376,10 @@ struct UniformF32 {
 struct UniformF64 {
     using value_type = double;
     static constexpr bool kHeavy = false;
-    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1) { return unit_double(next_d(s0, s1)); }
+    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1, const bm::LogTable * = nullptr)
+    {
+        return unit_double(next_d(s0, s1));
+    }
 };
 // Box-Muller, cosine branch.  The float32 variant works in float32 throughout;
 // log and cos are evaluated in double and rounded once, which is the closest
@@ -354,14 +387,14 @@ struct UniformF64 {
 struct NormalF32 {
     using value_type = float;
     static constexpr bool kHeavy = true;
-    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1)
+    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1, const bm::LogTable *tab)
     {
         const float u1 = UniformF32::draw(s0, s1);
         const float u2 = UniformF32::draw(s0, s1);
         const float two_pi = 6.283185307179586f;
-        const float lg = (float)log((double)u1);
+        const float lg = (float)bm::bm_log_f32(u1, tab);
         const float r = sqrtf(-2.0f * lg);
-        const float c = (float)cos((double)(two_pi * u2));
+        const float c = (float)bm::bm_cos_2pi((double)(two_pi * u2));
         return r * c;
     }
 };
@@ -370,14 +403,14 @@ struct NormalF32 {
 struct NormalF64 {
     using value_type = double;
     static constexpr bool kHeavy = true;
-    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1)
+    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1, const bm::LogTable *tab)
     {
         const float u1 = UniformF32::draw(s0, s1);
         const float u2 = UniformF32::draw(s0, s1);
         const double two_pi = 6.283185307179586;
-        const float lg = (float)log((double)u1);
+        const float lg = (float)bm::bm_log_f32(u1, tab);
         const double r = sqrt(-2.0 * (double)lg);
-        const double c = cos(two_pi * (double)u2);
+        const double c = bm::bm_cos_2pi(two_pi * (double)u2);
         return r * c;
     }
 };
@@ -402,13 +435,24 @@ template <typename VT> struct __attribute__((packed, aligned(sizeof(VT)))) OutPa
 template <typename Gen>
 __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__ states, int64_t n,
                                                           typename Gen::value_type *__restrict__ out,
-                                                          int64_t count)
+                                                          int64_t count, const bm::LogTable *__restrict__ log_table)
 {
     using VT = typename Gen::value_type;
     constexpr int ROUND = 128 / (int)sizeof(VT);  // values per generator per round
     constexpr int PER = 16 / (int)sizeof(VT);     // values per 16-byte packet
     constexpr int PITCH = ROUND + PER;            // 144-byte rows
     __shared__ __attribute__((aligned(16))) VT park_all[kFillBlock / 64][64][PITCH];
+
+    // the normal generators look their logarithm up in a 3 KiB table: into LDS first
+    __shared__ typename std::conditional<Gen::kHeavy, bm::LogTable, char>::type tab_store;
+    const bm::LogTable *tab = reinterpret_cast<const bm::LogTable *>(&tab_store);
+    if (Gen::kHeavy) {
+        const double *src = reinterpret_cast<const double *>(log_table);
+        double *dst = reinterpret_cast<double *>(&tab_store);
+        for (int k = threadIdx.x; k < (int)(sizeof(bm::LogTable) / sizeof(double)); k += kFillBlock)
+            dst[k] = src[k];
+        __syncthreads();
+    }
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -440,7 +484,7 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
                 } mine;
 #pragma unroll
                 for (int j = 0; j < ROUND; ++j)
-                    mine.val[j] = Gen::draw(s0, s1);
+                    mine.val[j] = Gen::draw(s0, s1, nullptr);
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
                     *reinterpret_cast<u32x4 *>(&park[lane][k * PER]) = mine.pk[k];
@@ -450,7 +494,7 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
             // inlined log/cos bodies only thrashes the instruction cache
 #pragma unroll 1
             for (int j = 0; j < m; ++j)
-                park[lane][j] = Gen::draw(s0, s1);
+                park[lane][j] = Gen::draw(s0, s1, tab);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -494,8 +538,14 @@ int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t 
     const int64_t grid = (n + kFillBlock - 1) / kFillBlock;
     if (grid > 0x7fffffffLL)
         return (int)hipErrorInvalidValue;
+    const bm::LogTable *log_table = nullptr;
+    if (Gen::kHeavy) {
+        int rc = device_log_table(&log_table);
+        if (rc)
+            return rc;
+    }
     hipLaunchKernelGGL((fill_kernel<Gen>), dim3((unsigned)grid), dim3(kFillBlock), 0, nbh_hip_stream(stream),
-                       (uint64_t *)states, n, (typename Gen::value_type *)out, count);
+                       (uint64_t *)states, n, (typename Gen::value_type *)out, count, log_table);
     return nbh_launch_status();
 }
 

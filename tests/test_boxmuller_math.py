@@ -1,0 +1,43 @@
+"""Host-side sweep of the Box-Muller logarithm and cosine (numba_cuda_amd/csrc/
+boxmuller_math.h) against long double: the same source the GPU kernels compile, built
+here with g++.  What is checked is independent of the oracle: x87 `logl` / `cosl`
+carry 64 bits, eleven more than the routines under test produce."""
+import os
+import re
+import subprocess
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(os.path.dirname(HERE), "numba_cuda_amd", "csrc")
+
+
+@pytest.fixture(scope="module")
+def sweep(tmp_path_factory):
+    exe = str(tmp_path_factory.mktemp("bm") / "check")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-I", CSRC,
+                    os.path.join(HERE, "boxmuller_math_check.cpp"), "-o", exe], check=True)
+    # every 7th mantissa: 1.2 M logarithms per binade and 2.4 M cosines per variant in ~1.5 s
+    out = subprocess.run([exe, "7"], check=True, capture_output=True, text=True).stdout
+    return out
+
+
+def test_logarithm_is_within_one_ulp_and_rounds_to_the_right_float32(sweep):
+    rows = re.findall(r"log binade 2\^-(\d+): n=(\d+) worst_ulp=([\d.]+) float_flips=(\d+)", sweep)
+    assert [int(r[0]) for r in rows] == [1, 2, 3, 24, 53]
+    for _, n, worst, flips in rows:
+        assert int(n) > 1_000_000
+        assert float(worst) <= 0.52          # tolerance: 0.52 ulp of the double result
+        assert int(flips) == 0
+    assert "log(1)=0 signbit=0 log(0)=-inf" in sweep
+
+
+def test_cosine_is_within_one_ulp(sweep):
+    rows = re.findall(r"cos variant (f\d+): n=(\d+) worst_ulp=([\d.]+) float_flips=(\d+)", sweep)
+    assert [r[0] for r in rows] == ["f64", "f32"]
+    for _, n, worst, flips in rows:
+        assert int(n) > 2_000_000
+        assert float(worst) <= 0.80          # tolerance: 0.8 ulp of the double result
+        assert int(flips) == 0
+    tiny = re.search(r"cos tiny arguments: worst_ulp=([\d.]+)", sweep)
+    assert float(tiny.group(1)) <= 0.5
