@@ -41,6 +41,13 @@ MEASURED_TRAFFIC = {
     "rng_uniform_f32": 4831936398,
     # profiles/transpose_sheared_f64_12345x6789.txt: 1 026 969 245 B fetched + 670 744 593 B written
     "transpose_f64": 1697713838,
+    # profiles/hbm_counters_other_workloads.txt
+    "reduce_f32_max": 1073822046,
+    "reduce_f64_sum": 1073820062,
+    "reduce_i64_sum": 2147534810,
+    "transpose_i16": 1074008367,
+    "rng_normal_f64": 2684437180,
+    "rng_init": 269594109,
 }
 
 
@@ -58,12 +65,12 @@ def _event_timed_launches(cuda, stream, launch, reps):
     return start.elapsed_time(stop) / reps
 
 
-def _cpu_baseline_reduce(a_host, target_seconds=12.0):
+def _cpu_baseline_reduce(a_host, target_seconds=12.0, functor=lambda x, y: x + y):
     """The reference's CPU path for reduce (its simulator: a left fold through the
     Python functor, one call per element, single core by construction), timed on a
     bounded prefix of the same input."""
     from oracle import sim
-    red = sim.Reduce(lambda x, y: x + y)
+    red = sim.Reduce(functor)
     probe = a_host[:1 << 18]
     t0 = time.perf_counter()
     red(probe, init=0)
@@ -75,9 +82,52 @@ def _cpu_baseline_reduce(a_host, target_seconds=12.0):
     red(sample, init=0)
     dt = time.perf_counter() - t0
     return {"value": round(sample.nbytes / dt / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "first 2^%d float32 elements of the same input, simulator-style left fold "
-                      "(functools.reduce over NumPy scalars), %.1f s" % (n.bit_length() - 1, dt),
+            "sample": "first 2^%d %s elements of the same input, simulator-style left fold "
+                      "(functools.reduce over NumPy scalars), %.1f s" % (n.bit_length() - 1, a_host.dtype.name, dt),
             "elements_per_s": round(n / dt, 1), "host_cores_available": os.cpu_count()}
+
+
+def _cpu_baseline_transpose(shape, dtype):
+    """The simulator's transpose is a NumPy view (no data moves); what a user then
+    pays is the materialising copy.  Timed on the 256 x 256 case the configuration
+    names, repeated for about a second."""
+    from oracle import sim
+    a = np.random.default_rng(2).random((256, 256)).astype(dtype)
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < 1.0:
+        np.ascontiguousarray(sim.transpose(a))
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(2 * a.nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "256 x 256 %s, simulator transpose (NumPy view) + materialising copy, %d repetitions"
+                      % (np.dtype(dtype).name, reps),
+            "host_cores_available": os.cpu_count()}
+
+
+def _cpu_baseline_rng(name, nthreads=4096):
+    """The simulator's RNG: sequential jump chain, then per-thread draws, all in
+    Python over NumPy uint64 scalars, one core, for the 4096 generators the
+    configuration names (about 5 s for the chain, 3 s for the draws)."""
+    from oracle import sim
+    from oracle.cref import STATE_DTYPE
+    states = np.zeros(nthreads, dtype=STATE_DTYPE)
+    t0 = time.perf_counter()
+    sim.init_states(states, 42)
+    t_init = time.perf_counter() - t0
+    if name == "rng_init":
+        return {"value": round(16 * nthreads / t_init / 1e9, 9), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "%d states by the sequential jump chain in NumPy-scalar Python, %.1f s" % (nthreads, t_init),
+                "states_per_s": round(nthreads / t_init, 1), "host_cores_available": os.cpu_count()}
+    draw, count, size = ((sim.uniform_float32, 64, 4) if name == "rng_uniform_f32" else (sim.normal_float64, 16, 8))
+    t0 = time.perf_counter()
+    for t in range(nthreads):
+        for _ in range(count):
+            draw(states, t)
+    dt = time.perf_counter() - t0
+    return {"value": round(size * nthreads * count / dt / 1e9, 9), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d generators x %d draws in NumPy-scalar Python, %.1f s (state initialisation %.1f s not included)"
+                      % (nthreads, count, dt, t_init),
+            "outputs_per_s": round(nthreads * count / dt, 1), "host_cores_available": os.cpu_count()}
 
 
 def _workload(name, cuda):
@@ -190,7 +240,7 @@ def _workload(name, cuda):
                 s.synchronize()
 
         return dict(desc="4096 x (65536 fp32) row sums round-robin over 4 streams, seed 3", dtype="f32",
-                    algo_bytes=host.nbytes, units=rows, step=step, stream=streams[0], host=None,
+                    algo_bytes=host.nbytes, units=rows, step=step, stream=streams[0], host=host,
                     kernel="reduce_kernel", keep=(dm, out, streams, views, slots), calls_per_step=rows)
     raise SystemExit("unknown workload %s" % name)
 
@@ -236,8 +286,17 @@ def main():
                     "launch_us_avg": round(launch_ms * 1e3, 2), "launches_timed": args.steps}
 
     cpu = None
-    if args.workload == "reduce_f32_sum" and not args.no_cpu_baseline:
-        cpu = _cpu_baseline_reduce(w["host"])
+    if not args.no_cpu_baseline:
+        name = args.workload
+        if name.startswith("reduce_"):
+            is_max = name.endswith("max")
+            cpu = _cpu_baseline_reduce(w["host"], functor=(lambda x, y: max(x, y)) if is_max else (lambda x, y: x + y))
+        elif name == "batched_reduce":
+            cpu = _cpu_baseline_reduce(w["host"].reshape(-1))
+        elif name.startswith("transpose_"):
+            cpu = _cpu_baseline_transpose(None, w["dtype"])
+        elif name.startswith("rng_"):
+            cpu = _cpu_baseline_rng(name)
 
     line = {
         "metric": "achieved HBM GB/s (% of 8 TB/s) for cuda.reduce fp32 sum at 2^28 elems"

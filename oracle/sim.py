@@ -100,3 +100,26 @@ def uniform_float64(states, index):
 def uniform_float32(states, index):
     """random.py:152-169"""
     return np.float32(uniform_float64(states, index))
+
+
+_TWO_PI_F32 = np.float32(2 * np.pi)
+_TWO_PI_F64 = np.float64(2 * np.pi)
+
+
+def normal_float32(states, index):
+    """random.py:191-213 in object mode: `math.log` / `math.cos` / `math.sqrt` of a
+    NumPy float32 go through Python floats (float64 precision), so only the products
+    round to float32.  Parity unpinned: derivable from the source, not confirmable
+    without running the reference."""
+    import math
+    u1 = uniform_float32(states, index)
+    u2 = uniform_float32(states, index)
+    return math.sqrt(-np.float32(2.0) * math.log(u1)) * math.cos(_TWO_PI_F32 * u2)
+
+
+def normal_float64(states, index):
+    """random.py:216-238 in object mode (float32 uniforms, float64 arithmetic)."""
+    import math
+    u1 = uniform_float32(states, index)
+    u2 = uniform_float32(states, index)
+    return math.sqrt(-np.float64(2.0) * math.log(u1)) * math.cos(_TWO_PI_F64 * u2)

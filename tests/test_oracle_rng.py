@@ -202,3 +202,16 @@ def test_normal_precision_mix():
         assert abs(np.float32(z32) - n32[t]) <= 2 * np.spacing(np.abs(n32[t]))
         z64 = np.sqrt(-2.0 * np.float64(lg)) * np.cos(np.float64(2 * np.pi) * np.float64(u2))
         assert abs(z64 - n64[t]) <= 4 * np.spacing(np.abs(n64[t]))
+
+
+def test_simulator_flavour_normals_track_the_compiled_flavour():
+    """The simulator evaluates log/cos through Python floats (random.py:191-238 in
+    object mode); the compiled flavour takes a float32 logarithm.  Same uniforms, same
+    states afterwards, values equal to within a float32 rounding of log(u1)."""
+    st = cref.init_states(16, 7)
+    for kind, draw, tol in (("normal_f32", sim.normal_float32, 2e-6), ("normal_f64", sim.normal_float64, 2e-6)):
+        want, after = cref.fill(st, 3, kind)
+        mine = st.copy()
+        got = np.array([[draw(mine, t) for _ in range(3)] for t in range(16)]).reshape(-1)
+        np.testing.assert_array_equal(mine, after)          # two generator steps per normal
+        np.testing.assert_allclose(got, want, rtol=tol, atol=1e-7)
