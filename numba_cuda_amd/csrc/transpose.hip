@@ -1,6 +1,6 @@
 // nbh_transpose: out[j, i] = in[i, j] for items of any size and any byte strides.
 //
-// Two kernels:
+// Four kernels:
 //   * packets - item size 1, 2, 4, 8 or 16 bytes with unit inner stride on both
 //               sides (row strides free).  Every lane moves V x V items, V = 16 /
 //               itemsize: it loads one 16-byte packet from each of V consecutive
@@ -21,9 +21,13 @@
 //               lines it is far worse than cached access (16388-wide: 2.3 vs
 //               4.2 TB/s) because neighbouring packets no longer meet in L2, so the
 //               kernel is instantiated both ways and the host picks by alignment.
-//   * strided - everything else (records such as 28-byte items, element strides,
-//               negative strides): one lane per (item, chunk) with the output
-//               index fastest, so writes stay as dense as the layout allows.
+//   * sheared - the same item sizes when output rows do not start on 128-byte lines
+//               (described at the kernel).
+//   * records - any other item size up to 512 bytes with unit inner stride: tiles
+//               through LDS in chunks of the widest aligned power of two.
+//   * strided - everything else (element strides, negative strides, huge items): one
+//               lane per (item, chunk) with the output index fastest, so writes stay
+//               as dense as the layout allows.
 //
 // HBM roofline: every item is read once and written once, 2*rows*cols*itemsize.
 #include "common.h"
@@ -283,6 +287,95 @@ __global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__rest
     }
 }
 
+// Items of any other size (records, 12-byte strings, 16-byte items that are only
+// 8-byte aligned ...) with unit inner stride on both sides: a T x T tile of items goes
+// through LDS in chunks of G bytes, G being the widest power of two that divides the
+// item size, the row strides and both base addresses.  Consecutive lanes read
+// consecutive chunks of an input row segment (T * itemsize contiguous bytes) and
+// write consecutive chunks of an output row segment, whatever the item size; the
+// divisions by the two run lengths are multiplications by precomputed reciprocals
+// (exact for operands below 2^16).  Measured, 8192^2 items of 12 bytes: 4.2 TB/s,
+// against 1.6 TB/s with one lane per chunk straight from global memory, where every
+// 4-byte read of a wavefront comes from a different input row.
+struct RecordShape {
+    int32_t itemsize, tile, chunks_per_run, pitch;  // run = tile * itemsize bytes
+    uint32_t inv_chunks_per_run, inv_itemsize;      // floor(2^32 / d) + 1
+};
+
+// W = 16 when WIDE (both bases and both row strides are multiples of 16, and so is
+// a run): global memory is then moved 16 bytes per lane although items can only be
+// picked out of the tile G bytes at a time.  Index arithmetic, not memory, bounds this
+// kernel, so the fewer chunks the better (28-byte items: 2.9 -> 4.3 TB/s, 3-byte
+// items 1.2 -> 1.9); with 8-byte pieces it no longer pays (24-byte items: 5.0 -> 4.4)
+// and is not used.
+template <int G, bool WIDE>
+__global__ __launch_bounds__(kThreads) void transpose_records(const char *__restrict__ in, char *__restrict__ out,
+                                                               int64_t rows, int64_t cols, int64_t in_s0,
+                                                               int64_t out_s0, int64_t tiles_r, RecordShape sh)
+{
+    using Piece = typename ItemOf<G>::type;
+    constexpr int W = WIDE ? 16 : G;
+    constexpr int NP = W / G;  // pieces per chunk
+    union Chunk {
+        Piece piece[NP];
+        typename ItemOf<W>::type whole;
+    };
+    extern __shared__ __attribute__((aligned(16))) char record_tile[];
+    const int64_t tile_c = (int64_t)blockIdx.x / tiles_r;  // consecutive workgroups go along the output rows
+    const int64_t tile_r = (int64_t)blockIdx.x % tiles_r;
+    const int64_t R0 = tile_r * sh.tile, C0 = tile_c * sh.tile;
+    const int nrows = (int)((rows - R0 < sh.tile) ? rows - R0 : sh.tile);
+    const int ncols = (int)((cols - C0 < sh.tile) ? cols - C0 : sh.tile);
+    const int total = sh.tile * sh.chunks_per_run;
+
+    const char *src = in + R0 * in_s0 + C0 * sh.itemsize;
+    const int in_run = ncols * sh.itemsize;  // bytes of one input row inside the tile
+    for (int idx = threadIdx.x; idx < total; idx += kThreads) {
+        const int r = (int)__umulhi((uint32_t)idx, sh.inv_chunks_per_run);
+        const int b = (idx - r * sh.chunks_per_run) * W;
+        if (r >= nrows || b >= in_run)
+            continue;
+        const char *g = src + (int64_t)r * in_s0 + b;
+        char *l = record_tile + r * sh.pitch + b;
+        if (b + W <= in_run) {
+            *reinterpret_cast<typename ItemOf<W>::type *>(l) = *reinterpret_cast<const typename ItemOf<W>::type *>(g);
+        } else {  // the run ends inside this chunk (last columns of the matrix)
+            for (int k = 0; b + k * G < in_run; ++k)
+                reinterpret_cast<Piece *>(l)[k] = reinterpret_cast<const Piece *>(g)[k];
+        }
+    }
+    __syncthreads();
+    char *dst = out + C0 * out_s0 + R0 * sh.itemsize;
+    const int out_run = nrows * sh.itemsize;  // bytes of one output row inside the tile
+    for (int idx = threadIdx.x; idx < total; idx += kThreads) {
+        const int c = (int)__umulhi((uint32_t)idx, sh.inv_chunks_per_run);
+        const int b = (idx - c * sh.chunks_per_run) * W;
+        if (c >= ncols || b >= out_run)
+            continue;
+        int r = (int)__umulhi((uint32_t)b, sh.inv_itemsize);
+        int within = b - r * sh.itemsize;
+        const char *l = record_tile + c * sh.itemsize;
+        char *g = dst + (int64_t)c * out_s0 + b;
+        Chunk v;
+#pragma unroll
+        for (int k = 0; k < NP; ++k) {
+            if (b + k * G < out_run)
+                v.piece[k] = *reinterpret_cast<const Piece *>(l + r * sh.pitch + within);
+            within += G;
+            if (within >= sh.itemsize) {
+                within -= sh.itemsize;
+                ++r;
+            }
+        }
+        if (b + W <= out_run) {
+            *reinterpret_cast<typename ItemOf<W>::type *>(g) = v.whole;
+        } else {
+            for (int k = 0; b + k * G < out_run; ++k)
+                reinterpret_cast<Piece *>(g)[k] = v.piece[k];
+        }
+    }
+}
+
 // One lane per G-byte chunk of one item; chunk index fastest, then the output's
 // inner index, then its outer index.
 template <int G>
@@ -344,6 +437,38 @@ int launch_sheared(const void *in, void *out, int64_t rows, int64_t cols, int64_
 }
 
 template <int G>
+int launch_records(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
+                   int64_t itemsize, hipStream_t stream)
+{
+    RecordShape sh;
+    sh.itemsize = (int32_t)itemsize;
+    sh.tile = itemsize <= 32 ? 32 : itemsize <= 128 ? 16 : 8;  // about 32 KiB of LDS at most
+    const int run = sh.tile * sh.itemsize;
+    const uint64_t mix = (uint64_t)(uintptr_t)in | (uint64_t)(uintptr_t)out | (uint64_t)in_s0 | (uint64_t)out_s0 |
+                         (uint64_t)run;
+    const bool wide = G <= 4 && mix % 16 == 0;
+    const int w = wide ? 16 : G;
+    sh.chunks_per_run = run / w;
+    sh.pitch = run + 16;
+    sh.inv_chunks_per_run = (uint32_t)(0x100000000ull / (uint32_t)sh.chunks_per_run) + 1u;
+    sh.inv_itemsize = (uint32_t)(0x100000000ull / (uint32_t)sh.itemsize) + 1u;
+    const int64_t tiles_r = (rows + sh.tile - 1) / sh.tile;
+    const int64_t tiles_c = (cols + sh.tile - 1) / sh.tile;
+    const int64_t tiles = tiles_r * tiles_c;
+    if (tiles > 0x7fffffffLL)
+        return (int)hipErrorInvalidValue;
+    const size_t lds = (size_t)sh.tile * sh.pitch;
+    const dim3 grid((unsigned)tiles), block(kThreads);
+    if (wide)
+        hipLaunchKernelGGL((transpose_records<G, (G <= 4)>), grid, block, lds, stream, (const char *)in, (char *)out,
+                           rows, cols, in_s0, out_s0, tiles_r, sh);
+    else
+        hipLaunchKernelGGL((transpose_records<G, false>), grid, block, lds, stream, (const char *)in, (char *)out,
+                           rows, cols, in_s0, out_s0, tiles_r, sh);
+    return nbh_launch_status();
+}
+
+template <int G>
 int launch_strided(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t in_s1,
                    int64_t out_s0, int64_t out_s1, int64_t itemsize, hipStream_t stream)
 {
@@ -400,6 +525,15 @@ extern "C" int nbh_transpose(const void *in, void *out, int64_t rows, int64_t co
         case 8: return launch_packets<8>(in, out, rows, cols, in_s0, out_s0, s);
         case 16: return launch_packets<16>(in, out, rows, cols, in_s0, out_s0, s);
         default: break;
+        }
+    }
+    if (unit_inner && itemsize <= 512) {
+        switch (g) {
+        case 1: return launch_records<1>(in, out, rows, cols, in_s0, out_s0, itemsize, s);
+        case 2: return launch_records<2>(in, out, rows, cols, in_s0, out_s0, itemsize, s);
+        case 4: return launch_records<4>(in, out, rows, cols, in_s0, out_s0, itemsize, s);
+        case 8: return launch_records<8>(in, out, rows, cols, in_s0, out_s0, itemsize, s);
+        default: return launch_records<16>(in, out, rows, cols, in_s0, out_s0, itemsize, s);
         }
     }
     switch (g) {

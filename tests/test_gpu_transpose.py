@@ -103,6 +103,29 @@ def test_every_item_size_and_ragged_shapes(shape, dtype):
     assert _same_bytes(got, cref.transpose(a))
 
 
+@pytest.mark.parametrize("itemsize", [3, 5, 6, 12, 20, 24, 28, 33, 100, 128, 200, 512, 520])
+def test_record_items_of_any_size(itemsize):
+    """Tile edge, chunk width and fallback all depend on the item size: below 33 bytes,
+    below 129, below 513, above."""
+    dtype = np.dtype("V%d" % itemsize)
+    for shape in ((70, 45), (1, 130), (257, 3)):
+        _say("transpose records", itemsize, shape)
+        raw = np.random.default_rng(itemsize).integers(0, 256, shape[0] * shape[1] * itemsize, dtype=np.uint8)
+        a = raw.view(dtype).reshape(shape)
+        got = cuda.to_device(a).T.copy_to_host()
+        assert got.shape == (shape[1], shape[0])
+        assert _same_bytes(got, np.ascontiguousarray(a.T))
+
+
+def test_sixteen_byte_items_that_are_only_eight_byte_aligned():
+    a = (np.arange(90 * 64) + 1j * np.arange(90 * 64)[::-1]).reshape(90, 64)
+    flat = cuda.to_device(np.zeros(90 * 64 * 2 + 1))
+    src = flat[1:].view(np.complex128).reshape(90, 64)       # base address = 8 mod 16
+    src.copy_to_device(a)
+    assert src.device_ctypes_pointer.value % 16 == 8
+    np.testing.assert_array_equal(transpose(src).copy_to_host(), a.T)
+
+
 def test_row_padded_inputs_and_outputs():
     """Rows longer than the logical width on both sides (pitched allocations)."""
     rng = np.random.default_rng(9)
