@@ -4,8 +4,13 @@
 // The host first squeezes the index space: axes of length 1 vanish and neighbouring
 // axes that are laid out back to back on both sides fuse.  What is left decides
 // the kernel:
-//   * one axis with unit stride on both sides -> a flat copy: 16-byte packets,
-//     grid-stride, the ragged tail done item by item
+//   * one axis with unit stride on both sides -> a flat copy: every workgroup owns
+//     a contiguous slice and streams it in 16-byte packets, four loads in flight per
+//     lane, non-temporal on both sides; packets start at the first 128-byte line of
+//     the destination, the bytes in front of it and behind the last packet are done
+//     chunk by chunk.  Measured on MI355X, 2^28 float32: grid-stride cached packets
+//     4.80 TB/s, non-temporal 5.03, contiguous slices + non-temporal 5.48
+//     (hipMemcpyDtoD: 5.2)
 //   * anything else -> one lane per chunk of an item, innermost axis fastest
 //
 // HBM roofline of the flat copy: bytes read + bytes written = 2 * n * itemsize.
@@ -27,22 +32,44 @@ template <> struct ChunkOf<8> { using type = uint64_t; };
 template <> struct ChunkOf<16> { using type = Chunk16; };
 
 // 16 bytes that are only aligned to G
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <int G> struct __attribute__((packed, aligned(G))) Packet {
-    typename ChunkOf<G>::type c[16 / G];
+    u32x4 v;
 };
 
 template <int G>
 __global__ __launch_bounds__(kThreads) void copy_flat(char *__restrict__ dst, const char *__restrict__ src,
-                                                      int64_t nbytes)
+                                                      int64_t nbytes, int64_t head)
 {
-    const int64_t npack = nbytes / 16;
-    const int64_t step = (int64_t)gridDim.x * kThreads;
-    const int64_t first = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    for (int64_t i = first; i < npack; i += step)
-        *reinterpret_cast<Packet<G> *>(dst + i * 16) = *reinterpret_cast<const Packet<G> *>(src + i * 16);
-    using C = typename ChunkOf<G>::type;
-    for (int64_t b = npack * 16 + first * G; b < nbytes; b += step * G)
-        *reinterpret_cast<C *>(dst + b) = *reinterpret_cast<const C *>(src + b);
+    constexpr int kInFlight = 4;
+    const int64_t npack = (nbytes - head) / 16;
+    const Packet<G> *__restrict__ from = reinterpret_cast<const Packet<G> *>(src + head);
+    Packet<G> *__restrict__ to = reinterpret_cast<Packet<G> *>(dst + head);
+    const int64_t per = (npack + gridDim.x - 1) / gridDim.x;
+    const int64_t begin = (int64_t)blockIdx.x * per;
+    int64_t end = begin + per;
+    if (end > npack)
+        end = npack;
+    int64_t i = begin + threadIdx.x;
+    for (; i + (kInFlight - 1) * kThreads < end; i += kInFlight * kThreads) {
+        u32x4 v[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+            v[u] = __builtin_nontemporal_load(&from[i + u * kThreads].v);
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+            __builtin_nontemporal_store(v[u], &to[i + u * kThreads].v);
+    }
+    for (; i < end; i += kThreads)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(&from[i].v), &to[i].v);
+
+    if (blockIdx.x == 0) {  // fewer than 128 + 16 bytes in all
+        using C = typename ChunkOf<G>::type;
+        for (int64_t b = (int64_t)threadIdx.x * G; b < head; b += (int64_t)kThreads * G)
+            *reinterpret_cast<C *>(dst + b) = *reinterpret_cast<const C *>(src + b);
+        for (int64_t b = head + npack * 16 + (int64_t)threadIdx.x * G; b < nbytes; b += (int64_t)kThreads * G)
+            *reinterpret_cast<C *>(dst + b) = *reinterpret_cast<const C *>(src + b);
+    }
 }
 
 struct Dims {
@@ -75,14 +102,18 @@ inline int64_t low_bit(uint64_t x) { return (int64_t)(x & (~x + 1)); }
 
 template <int G> int launch_flat(void *dst, const void *src, int64_t nbytes, hipStream_t s)
 {
-    int64_t grid = (nbytes / 16 + kThreads - 1) / kThreads;
+    // bytes in front of the destination's first 128-byte line (a multiple of G)
+    int64_t head = (int64_t)((128 - (uintptr_t)dst % 128) % 128);
+    if (head > nbytes)
+        head = nbytes;
+    int64_t grid = ((nbytes - head) / 16 + 4 * kThreads - 1) / (4 * kThreads);
     const int64_t cap = (int64_t)nbh_cu_count() * 8;
     if (grid > cap)
         grid = cap;
     if (grid < 1)
         grid = 1;
     hipLaunchKernelGGL((copy_flat<G>), dim3((unsigned)grid), dim3(kThreads), 0, s, (char *)dst, (const char *)src,
-                       nbytes);
+                       nbytes, head);
     return nbh_launch_status();
 }
 

@@ -65,6 +65,24 @@ def test_cuda_array_interface_with_torch_tensors():
         cuda.as_cuda_array(np.zeros(3))
 
 
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float32, np.complex128])
+def test_flat_assignment_at_every_alignment(dtype):
+    """dst[a:a+n] = src[b:b+n]: the copy kernel starts its 16-byte packets at the
+    destination's first 128-byte line; what lies in front and behind goes item by item."""
+    rng = np.random.default_rng(11)
+    size = 140000
+    src_host = rng.integers(0, 255, size * np.dtype(dtype).itemsize, dtype=np.uint8).view(dtype)
+    src = cuda.to_device(src_host)
+    for n in (1, 7, 31, 32, 33, 127, 128, 129, 1000, 4099, 100003):
+        for d_off, s_off in ((0, 0), (1, 0), (0, 3), (5, 9), (37, 64)):
+            want = np.zeros(size, dtype)
+            dst = cuda.to_device(want)
+            dst[d_off:d_off + n] = src[s_off:s_off + n]
+            want[d_off:d_off + n] = src_host[s_off:s_off + n]
+            got = dst.copy_to_host()
+            assert got.tobytes() == want.tobytes(), (n, d_off, s_off)
+
+
 def test_setitem_scalars_rows_columns_broadcast():
     """`darr[key] = value` (reference: tests/cudadrv/test_cuda_array_slicing.py:220-379)."""
     a = np.arange(5 * 7, dtype=np.float64).reshape(5, 7)
