@@ -505,7 +505,8 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
                 const int l = k * 8 + row;
                 if (l < lanes_here) {
                     u32x4 v = *reinterpret_cast<const u32x4 *>(&park[l][sub * PER]);
-                    reinterpret_cast<OutPacket<VT> *>(base + (int64_t)l * count + i0 + sub * PER)->v = v;
+                    __builtin_nontemporal_store(
+                        v, &reinterpret_cast<OutPacket<VT> *>(base + (int64_t)l * count + i0 + sub * PER)->v);
                 }
             }
         } else {
