@@ -83,6 +83,45 @@ def test_flat_assignment_at_every_alignment(dtype):
             assert got.tobytes() == want.tobytes(), (n, d_off, s_off)
 
 
+@pytest.mark.parametrize("dtype", [np.uint8, np.float32, np.complex128])
+def test_block_assignment_in_pitched_arrays(dtype):
+    """dst[r0:r1, c0:c1] = src[...]: rows are runs of bytes at whatever alignment the
+    slice gives them; also rows shorter than a packet, a broadcast row, and 3-D blocks."""
+    rng = np.random.default_rng(12)
+    item = np.dtype(dtype).itemsize
+
+    def rand(shape):
+        return rng.integers(0, 255, int(np.prod(shape)) * item, dtype=np.uint8).view(dtype).reshape(shape)
+
+    src_host = rand((300, 700))
+    src = cuda.to_device(src_host)
+    for (r0, r1, c0, c1, sr, sc) in ((0, 300, 0, 700, 0, 0), (3, 290, 5, 650, 1, 7), (10, 11, 1, 2, 0, 0),
+                                     (0, 300, 699, 700, 0, 3), (7, 207, 33, 36, 50, 100), (1, 256, 16, 528, 2, 32)):
+        want = np.zeros((300, 700), dtype)
+        dst = cuda.to_device(want)
+        h, w = r1 - r0, c1 - c0
+        dst[r0:r1, c0:c1] = src[sr:sr + h, sc:sc + w]
+        want[r0:r1, c0:c1] = src_host[sr:sr + h, sc:sc + w]
+        assert dst.copy_to_host().tobytes() == want.tobytes(), (r0, r1, c0, c1, sr, sc)
+    # one row broadcast down a block
+    want = np.zeros((300, 700), dtype)
+    dst = cuda.to_device(want)
+    dst[5:205, 9:409] = src[17, 3:403]
+    want[5:205, 9:409] = src_host[17, 3:403]
+    assert dst.copy_to_host().tobytes() == want.tobytes()
+    # three axes that do not fuse
+    cube_host = rand((20, 30, 40))
+    cube = cuda.to_device(cube_host)
+    want = np.zeros((20, 30, 40), dtype)
+    dst = cuda.to_device(want)
+    dst[1:19, 2:29, 3:39] = cube[0:18, 1:28, 4:40]
+    want[1:19, 2:29, 3:39] = cube_host[0:18, 1:28, 4:40]
+    assert dst.copy_to_host().tobytes() == want.tobytes()
+    dst[2:4, :, 8:24] = cube[5:7, :, 16:32]
+    want[2:4, :, 8:24] = cube_host[5:7, :, 16:32]
+    assert dst.copy_to_host().tobytes() == want.tobytes()
+
+
 def test_setitem_scalars_rows_columns_broadcast():
     """`darr[key] = value` (reference: tests/cudadrv/test_cuda_array_slicing.py:220-379)."""
     a = np.arange(5 * 7, dtype=np.float64).reshape(5, 7)
