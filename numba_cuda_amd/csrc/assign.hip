@@ -205,6 +205,18 @@ int launch_strided(void *dst, const void *src, const Dims &d, int64_t itemsize, 
 
 }  // namespace
 
+int nbh_flat_copy(void *dst, const void *src, int64_t nbytes, hipStream_t stream)
+{
+    const uint64_t mix = (uint64_t)(uintptr_t)dst | (uint64_t)(uintptr_t)src | (uint64_t)nbytes | 16u;
+    switch (low_bit(mix)) {
+    case 1: return launch_flat<1>(dst, src, nbytes, stream);
+    case 2: return launch_flat<2>(dst, src, nbytes, stream);
+    case 4: return launch_flat<4>(dst, src, nbytes, stream);
+    case 8: return launch_flat<8>(dst, src, nbytes, stream);
+    default: return launch_flat<16>(dst, src, nbytes, stream);
+    }
+}
+
 extern "C" int nbh_assign(void *dst, const void *src, int ndim, const int64_t *shape, const int64_t *dst_strides,
                           const int64_t *src_strides, int64_t itemsize, nbh_stream_t stream)
 {

@@ -21,3 +21,7 @@ static inline hipStream_t nbh_hip_stream(nbh_stream_t s) { return (hipStream_t)s
 
 // Number of compute units of the current device (cached per device).
 int nbh_cu_count();
+
+// dst[0:nbytes] = src[0:nbytes] with the flat copy kernel of nbh_assign, on `stream`
+// (asynchronous).  Both ranges must be memory the current device can address.
+int nbh_flat_copy(void *dst, const void *src, int64_t nbytes, hipStream_t stream);

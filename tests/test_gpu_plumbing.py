@@ -83,6 +83,30 @@ def test_flat_assignment_at_every_alignment(dtype):
             assert got.tobytes() == want.tobytes(), (n, d_off, s_off)
 
 
+def test_large_device_to_device_copies():
+    """copy_to_device between device arrays of a MiB and more runs on the library's own
+    copy kernel (smaller ones on hipMemcpy): with and without a stream, at odd offsets."""
+    rng = np.random.default_rng(13)
+    host = rng.integers(0, 255, (1 << 22) + 77, dtype=np.uint8)
+    src = cuda.to_device(host)
+    st = cuda.stream()
+    for lo, n in ((0, 1 << 22), (3, (1 << 21) + 5), (129, (1 << 20)), (1, (1 << 20) - 1), (0, 100)):
+        dst = cuda.device_array(n + 64, np.uint8)
+        dst.gpu_data.memset(0)
+        dst[16:16 + n].copy_to_device(src[lo:lo + n])
+        got = dst.copy_to_host()
+        assert got[16:16 + n].tobytes() == host[lo:lo + n].tobytes() and not got[:16].any() and not got[16 + n:].any()
+        dst2 = cuda.device_array(n, np.uint8)
+        dst2.copy_to_device(src[lo:lo + n], stream=st)
+        st.synchronize()
+        assert dst2.copy_to_host().tobytes() == host[lo:lo + n].tobytes()
+    m = cuda.mapped_array(1 << 21, np.uint8)          # not plain device memory: hipMemcpy's business
+    m[:] = host[:1 << 21]
+    d = cuda.device_array(1 << 21, np.uint8)
+    d.copy_to_device(m)
+    assert d.copy_to_host().tobytes() == host[:1 << 21].tobytes()
+
+
 @pytest.mark.parametrize("dtype", [np.uint8, np.float32, np.complex128])
 def test_block_assignment_in_pitched_arrays(dtype):
     """dst[r0:r1, c0:c1] = src[...]: rows are runs of bytes at whatever alignment the
