@@ -38,11 +38,7 @@ template <> struct ChunkOf<4> { using type = uint32_t; };
 template <> struct ChunkOf<8> { using type = uint64_t; };
 template <> struct ChunkOf<16> { using type = Chunk16; };
 
-// 16 bytes that are only aligned to G
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-template <int G> struct __attribute__((packed, aligned(G))) Packet {
-    u32x4 v;
-};
+typedef nbh_u32x4 u32x4;
 
 template <int G>
 __global__ __launch_bounds__(kThreads) void copy_flat(char *__restrict__ dst, const char *__restrict__ src,
@@ -50,18 +46,18 @@ __global__ __launch_bounds__(kThreads) void copy_flat(char *__restrict__ dst, co
 {
     constexpr int kInFlight = 4;
     const int64_t npack = (nbytes - head) / 16;
-    const Packet<G> *__restrict__ from = reinterpret_cast<const Packet<G> *>(src + head);
-    Packet<G> *__restrict__ to = reinterpret_cast<Packet<G> *>(dst + head);
+    const char *__restrict__ from = src + head;  // packets: G-aligned here,
+    char *__restrict__ to = dst + head;           // 128-byte aligned here
     const int64_t p0 = (int64_t)blockIdx.x * (kThreads * kInFlight) + threadIdx.x;
     u32x4 v[kInFlight];
 #pragma unroll
     for (int u = 0; u < kInFlight; ++u)
         if (p0 + u * kThreads < npack)
-            v[u] = __builtin_nontemporal_load(&from[p0 + u * kThreads].v);
+            v[u] = nbh_load16<G, true>(from + (p0 + u * kThreads) * 16);
 #pragma unroll
     for (int u = 0; u < kInFlight; ++u)
         if (p0 + u * kThreads < npack)
-            __builtin_nontemporal_store(v[u], &to[p0 + u * kThreads].v);
+            nbh_store16<16, true>(to + (p0 + u * kThreads) * 16, v[u]);
 
     if (blockIdx.x == 0) {  // fewer than 128 + 16 bytes in all
         using C = typename ChunkOf<G>::type;
@@ -94,21 +90,14 @@ __global__ __launch_bounds__(kThreads) void copy_rows(char *__restrict__ dst, co
 #pragma unroll
     for (int u = 0; u < kInFlight; ++u) {
         const int64_t p = p0 + (int64_t)u * tx_count;
-        if (p < npack) {
-            const Packet<G> *q = reinterpret_cast<const Packet<G> *>(from + p * 16);
-            v[u] = NT ? __builtin_nontemporal_load(&q->v) : q->v;
-        }
+        if (p < npack)
+            v[u] = nbh_load16<G, NT>(from + p * 16);
     }
 #pragma unroll
     for (int u = 0; u < kInFlight; ++u) {
         const int64_t p = p0 + (int64_t)u * tx_count;
-        if (p < npack) {
-            Packet<G> *q = reinterpret_cast<Packet<G> *>(to + p * 16);
-            if (NT)
-                __builtin_nontemporal_store(v[u], &q->v);
-            else
-                q->v = v[u];
-        }
+        if (p < npack)
+            nbh_store16<G, NT>(to + p * 16, v[u]);
     }
     if (seg == segs - 1) {  // fewer than 16 bytes behind the last packet
         using C = typename ChunkOf<G>::type;

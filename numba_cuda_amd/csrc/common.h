@@ -25,3 +25,29 @@ int nbh_cu_count();
 // dst[0:nbytes] = src[0:nbytes] with the flat copy kernel of nbh_assign, on `stream`
 // (asynchronous).  Both ranges must be memory the current device can address.
 int nbh_flat_copy(void *dst, const void *src, int64_t nbytes, hipStream_t stream);
+
+// Sixteen bytes at an address that is only A-byte aligned, moved as one vector:
+// global memory takes 128-bit accesses at any alignment, and the under-aligned
+// vector type tells the compiler exactly what it may assume.  NT = non-temporal.
+typedef uint32_t nbh_u32x4 __attribute__((ext_vector_type(4)));
+template <int A> struct nbh_packet;
+template <> struct nbh_packet<1> { typedef nbh_u32x4 type __attribute__((aligned(1))); };
+template <> struct nbh_packet<2> { typedef nbh_u32x4 type __attribute__((aligned(2))); };
+template <> struct nbh_packet<4> { typedef nbh_u32x4 type __attribute__((aligned(4))); };
+template <> struct nbh_packet<8> { typedef nbh_u32x4 type __attribute__((aligned(8))); };
+template <> struct nbh_packet<16> { typedef nbh_u32x4 type __attribute__((aligned(16))); };
+template <int A, bool NT> __device__ __forceinline__ nbh_u32x4 nbh_load16(const void *p)
+{
+    const typename nbh_packet<A>::type *q = static_cast<const typename nbh_packet<A>::type *>(p);
+    if (NT)
+        return __builtin_nontemporal_load(q);
+    return *q;
+}
+template <int A, bool NT> __device__ __forceinline__ void nbh_store16(void *p, nbh_u32x4 v)
+{
+    typename nbh_packet<A>::type *q = static_cast<typename nbh_packet<A>::type *>(p);
+    if (NT)
+        __builtin_nontemporal_store(v, q);
+    else
+        *q = v;
+}

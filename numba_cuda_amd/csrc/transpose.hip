@@ -46,13 +46,9 @@ template <> struct ItemOf<4> { using type = uint32_t; };
 template <> struct ItemOf<8> { using type = uint64_t; };
 template <> struct ItemOf<16> { using type = Item16; };
 
-// Sixteen bytes as a vector the compiler can load / store with one instruction,
-// non-temporally, at any item-aligned address (global memory accepts 128-bit
-// accesses that are only item-aligned).
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-template <int E> struct __attribute__((packed, aligned(E))) Packet {
-    u32x4 v;
-};
+// Sixteen bytes as one vector: loaded / stored with one instruction at any
+// item-aligned address (nbh_load16 / nbh_store16).
+typedef nbh_u32x4 u32x4;
 
 // Shape of the workgroup tile per item size: WR x WC wavefronts, REP wavefront
 // tiles stacked along the rows per wavefront.  A wavefront tile is 8V x 8V items.
@@ -79,8 +75,7 @@ __device__ __forceinline__ void move_block(const char *__restrict__ in, char *__
     for (int j = 0; j < V; ++j) {
         const char *src = in + (r0 + j) * in_s0 + c0 * E;
         if (!GUARD || (r0 + j < rows && c0 + V <= cols)) {
-            const Packet<E> *p = reinterpret_cast<const Packet<E> *>(src);
-            a.pk[j] = NT ? __builtin_nontemporal_load(&p->v) : p->v;
+            a.pk[j] = nbh_load16<E, NT>(src);
         } else if (r0 + j < rows) {
             for (int k = 0; k < V; ++k)
                 if (c0 + k < cols)
@@ -96,11 +91,7 @@ __device__ __forceinline__ void move_block(const char *__restrict__ in, char *__
     for (int i = 0; i < V; ++i) {
         char *dst = out + (c0 + i) * out_s0 + r0 * E;
         if (!GUARD || (c0 + i < cols && r0 + V <= rows)) {
-            Packet<E> *p = reinterpret_cast<Packet<E> *>(dst);
-            if (NT)
-                __builtin_nontemporal_store(b.pk[i], &p->v);
-            else
-                p->v = b.pk[i];
+            nbh_store16<E, NT>(dst, b.pk[i]);
         } else if (c0 + i < cols) {
             for (int k = 0; k < V; ++k)
                 if (r0 + k < rows)
@@ -175,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__rest
     constexpr int NL = TR / L + 2;  // lines of one output row a step can touch, at most
     __shared__ Item ring[RING][TC + ShearOf<E>::PAD];
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x;
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  When a
     // tile row is no wider than a line and input rows straddle lines, neighbouring
     // column bands fetch the same lines: give each XCD a contiguous share of the bands
@@ -217,7 +208,7 @@ __global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__rest
                 continue;
             const char *src = in + gr * in_s0 + gc * E;
             if (gc + V <= cols) {
-                held[k].pk = reinterpret_cast<const Packet<E> *>(src)->v;
+                held[k].pk = nbh_load16<E, false>(src);
             } else {
                 for (int j = 0; j < V; ++j)
                     if (gc + j < cols)
@@ -380,9 +371,9 @@ __global__ __launch_bounds__(kThreads) void transpose_records(const char *__rest
 // inner index, then its outer index.
 template <int G>
 __global__ __launch_bounds__(kThreads) void transpose_strided(const char *__restrict__ in, char *__restrict__ out,
-                                                               int64_t rows, int64_t cols, int64_t in_s0,
-                                                               int64_t in_s1, int64_t out_s0, int64_t out_s1,
-                                                               int64_t chunks, int64_t total)
+                                                               int64_t rows, int64_t in_s0, int64_t in_s1,
+                                                               int64_t out_s0, int64_t out_s1, int64_t chunks,
+                                                               int64_t total)
 {
     using Chunk = typename ItemOf<G>::type;
     const int64_t step = (int64_t)gridDim.x * kThreads;
@@ -479,7 +470,7 @@ int launch_strided(const void *in, void *out, int64_t rows, int64_t cols, int64_
     if (grid > cap)
         grid = cap;
     hipLaunchKernelGGL((transpose_strided<G>), dim3((unsigned)grid), dim3(kThreads), 0, stream, (const char *)in,
-                       (char *)out, rows, cols, in_s0, in_s1, out_s0, out_s1, chunks, total);
+                       (char *)out, rows, in_s0, in_s1, out_s0, out_s1, chunks, total);
     return nbh_launch_status();
 }
 

@@ -417,12 +417,9 @@ struct NormalF64 {
 
 constexpr int kFillBlock = 256;
 
-// 16 bytes of output values that are only guaranteed the alignment of one value
-// (runs start at t*count, which need not be a multiple of four values).
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-template <typename VT> struct __attribute__((packed, aligned(sizeof(VT)))) OutPacket {
-    u32x4 v;
-};
+// Output packets of 16 bytes are only guaranteed the alignment of one value (runs
+// start at t*count, which need not be a multiple of four values): nbh_store16.
+typedef nbh_u32x4 u32x4;
 
 // Each wavefront works on its own 64 generators and its own slice of LDS, so
 // wavefronts never wait for one another.  A round is 128 bytes per generator: the
@@ -505,8 +502,7 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
                 const int l = k * 8 + row;
                 if (l < lanes_here) {
                     u32x4 v = *reinterpret_cast<const u32x4 *>(&park[l][sub * PER]);
-                    __builtin_nontemporal_store(
-                        v, &reinterpret_cast<OutPacket<VT> *>(base + (int64_t)l * count + i0 + sub * PER)->v);
+                    nbh_store16<(int)sizeof(VT), true>(base + (int64_t)l * count + i0 + sub * PER, v);
                 }
             }
         } else {
