@@ -6,10 +6,10 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 import numba_cuda_amd as cuda
-from tests import plumbing_cases
+from tests import ndarray_cases, plumbing_cases
 
 
-@pytest.mark.parametrize("case", plumbing_cases.ALL, ids=lambda f: f.__name__)
+@pytest.mark.parametrize("case", plumbing_cases.ALL + ndarray_cases.ALL, ids=lambda f: f.__name__)
 def test_plumbing(case):
     print(case.__name__, flush=True)
     case(cuda)
