@@ -1,14 +1,19 @@
-"""Ahead-of-time build of libnbhip.so (the HIP back end) for gfx950.
+"""Ahead-of-time build of the two native parts of the package:
+
+    libnbhip.so   the HIP back end for gfx950 (hipcc)
+    _hostbuf      a small CPython extension: buffer protocol for host allocations and
+                  byte extents of strided buffers (gcc)
 
     python -m numba_cuda_amd._build
 
-There is no JIT in this package: the kernels are compiled once, here, with hipcc.
+There is no JIT in this package: everything is compiled once, here.
 """
 
 import os
 import shutil
 import subprocess
 import sys
+import sysconfig
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 SRC_DIR = os.path.join(PKG_DIR, "csrc")
@@ -28,6 +33,26 @@ HIPCC_FLAGS = [
     # keep the compiler from forming packed fp32 instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+
+
+HOSTBUF_SRC = os.path.join(PKG_DIR, "cext", "hostbuf.c")
+HOSTBUF_PATH = os.path.join(PKG_DIR, "_hostbuf" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_hostbuf(verbose=False):
+    """Compile cext/hostbuf.c into the extension module numba_cuda_amd._hostbuf."""
+    cc = os.environ.get("CC") or shutil.which("gcc") or shutil.which("cc")
+    if not cc:
+        raise RuntimeError("no C compiler found for numba_cuda_amd/cext/hostbuf.c (set CC)")
+    tmp = HOSTBUF_PATH + ".tmp"
+    cmd = [cc, "-O2", "-Wall", "-shared", "-fPIC", "-I", sysconfig.get_paths()["include"], HOSTBUF_SRC, "-o", tmp]
+    if verbose:
+        print(" ".join(cmd))
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building _hostbuf failed:\n" + proc.stdout)
+    os.replace(tmp, HOSTBUF_PATH)
+    return HOSTBUF_PATH
 
 
 def find_hipcc():
@@ -58,4 +83,5 @@ def build(verbose=False):
 
 
 if __name__ == "__main__":
+    print(build_hostbuf(verbose="-v" in sys.argv))
     print(build(verbose="-v" in sys.argv))

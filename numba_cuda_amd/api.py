@@ -81,7 +81,7 @@ def _pinned_ndarray(shape, dtype, strides, order, **alloc_flags):
     shape, strides, dtype = prepare_shape_strides_dtype(shape, strides, dtype, order)
     nbytes = driver.memory_size_from_info(shape, strides, dtype.itemsize)
     mem = _ctx().memhostalloc(nbytes, **alloc_flags)
-    ary = np.ndarray(shape=shape, strides=strides, dtype=dtype, order=order, buffer=mem.as_buffer())
+    ary = np.ndarray(shape=shape, strides=strides, dtype=dtype, order=order, buffer=mem)
     return ary, mem
 
 
@@ -119,7 +119,7 @@ def managed_array(shape, dtype=np.float64, strides=None, order="C", stream=0, at
     shape, strides, dtype = prepare_shape_strides_dtype(shape, strides, dtype, order)
     nbytes = driver.memory_size_from_info(shape, strides, dtype.itemsize)
     mem = _ctx().memallocmanaged(nbytes, attach_global=attach_global)
-    ary = np.ndarray(shape=shape, strides=strides, dtype=dtype, order=order, buffer=mem.as_buffer())
+    ary = np.ndarray(shape=shape, strides=strides, dtype=dtype, order=order, buffer=mem)
     out = np.ndarray.view(ary, type=devicearray.ManagedNDArray)
     out.device_setup(mem, stream=stream)
     return out

@@ -28,6 +28,13 @@ from ctypes import c_int, c_size_t, c_void_p, byref
 import numpy as np
 
 from numba_cuda_amd import _lib
+
+try:
+    from numba_cuda_amd import _hostbuf
+except ImportError:                      # not built yet: one gcc call, about a second
+    from numba_cuda_amd import _build
+    _build.build_hostbuf()
+    from numba_cuda_amd import _hostbuf
 from numba_cuda_amd.core import config
 from numba_cuda_amd.core.errors import CudaDriverError, CudaSupportError  # noqa: F401
 
@@ -720,15 +727,14 @@ class AutoFreePointer(MemoryPointer):
         self.refct -= 1
 
 
-class _HostBufferMixin:
-    """Gives NumPy a buffer over [host_pointer, host_pointer + size) that keeps the
-    allocation alive (the reference does this with a C extension type,
-    cext/mviewbuf.c:212-363)."""
+class _HostBufferMixin(_hostbuf.HostBuffer):
+    """Host-visible memory objects export [_bufptr_, _bufptr_ + _buflen_) through the
+    buffer protocol (`np.ndarray(shape, dtype, buffer=mem)`); the buffer keeps the
+    allocation alive.  The base class is native (cext/hostbuf.c), as the reference's is
+    (cext/mviewbuf.c:212-363)."""
 
     def as_buffer(self):
-        buf = (ctypes.c_byte * self.size).from_address(self.host_pointer)
-        buf._keepalive = self
-        return buf
+        return self
 
 
 class MappedMemory(AutoFreePointer, _HostBufferMixin):
@@ -805,6 +811,12 @@ class OwnedPointer:
     def __getattr__(self, fname):
         return getattr(self._view, fname)
 
+    def view(self, start, stop=None):
+        # a real method rather than a fall-through: in `ctx.memalloc(n).view(k)` the
+        # temporary reference must outlive the call, or the memory is freed before the
+        # derived pointer has taken its own reference
+        return self._view.view(start, stop)
+
 
 def _drop_reference(mem):
     try:
@@ -839,10 +851,6 @@ class Stream:
 
     def __int__(self):
         return self.handle
-
-    def __bool__(self):
-        # stream 0 is "no stream": copies on it are synchronous
-        return self.handle != 0
 
     def __eq__(self, other):
         if isinstance(other, Stream):
@@ -1005,23 +1013,13 @@ def host_pointer(obj, readonly=False):
         return obj.__array_interface__["data"][0]
     if isinstance(obj, ctypes.Array):
         return ctypes.addressof(obj)
-    mv = memoryview(obj)
-    if not readonly and mv.readonly:
-        raise BufferError("writable buffer requested from a read-only object")
-    return np.frombuffer(mv, dtype=np.uint8).ctypes.data if mv.nbytes else 0
+    return _hostbuf.address(obj, not readonly)
 
 
 def _extents(ptr, shape, strides, itemsize):
     """Half-open byte range an array touches (reference cext/mviewbuf.c:76-135)."""
-    lo = hi = ptr
-    for n, s in zip(shape, strides):
-        if n == 0:
-            return ptr, ptr
-        if s > 0:
-            hi += s * (n - 1)
-        elif s < 0:
-            lo += s * (n - 1)
-    return lo, hi + itemsize
+    lo, hi = _hostbuf.extents_of(shape, strides, itemsize)
+    return ptr + lo, ptr + hi
 
 
 def host_memory_extents(obj):
@@ -1029,9 +1027,7 @@ def host_memory_extents(obj):
     if isinstance(obj, (np.ndarray, np.generic)):
         a = np.asarray(obj)
         return _extents(a.__array_interface__["data"][0], a.shape, a.strides, a.itemsize)
-    mv = memoryview(obj)
-    strides = mv.strides if mv.strides is not None else ()
-    return _extents(host_pointer(obj, readonly=True), mv.shape, strides, mv.itemsize)
+    return _hostbuf.extents(obj)
 
 
 def host_memory_size(obj):

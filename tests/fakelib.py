@@ -143,6 +143,11 @@ class FakeLib:
                 self._out(base, addr)
                 self._out(size, len(buf) - (addr - ctypes.addressof(buf)))
                 return 0
+        for addr, buf in self.host_buffers.items():      # device-mapped host allocations
+            if addr <= a < addr + len(buf):
+                self._out(base, addr)
+                self._out(size, len(buf))
+                return 0
         return HIP_ERROR_INVALID_VALUE
 
     def _copy(self, kind, dst, src, nbytes, stream):

@@ -6,10 +6,13 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 import numba_cuda_amd as cuda
-from tests import ndarray_cases, plumbing_cases
+from tests import host_stream_cases, memory_cases, ndarray_cases, plumbing_cases, slicing_cases
+
+CASES = (plumbing_cases.ALL + ndarray_cases.ALL + slicing_cases.ALL + memory_cases.ALL
+         + host_stream_cases.ALL)
 
 
-@pytest.mark.parametrize("case", plumbing_cases.ALL + ndarray_cases.ALL, ids=lambda f: f.__name__)
+@pytest.mark.parametrize("case", CASES, ids=lambda f: f.__name__)
 def test_plumbing(case):
     print(case.__name__, flush=True)
     case(cuda)

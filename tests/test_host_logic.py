@@ -269,7 +269,9 @@ def test_stream_handle_rules():
     assert drv._stream_handle(drv.Stream(77)) == 77
     with pytest.raises(TypeError, match="Expected a Stream object or 0"):
         drv._stream_handle("s")
-    assert not drv.Stream(0) and drv.Stream(5)
+    # a Stream object is always "a stream was given", the default stream too (the
+    # reference's tests/cudadrv/test_cuda_array_slicing.py:341-379 depend on it)
+    assert drv.Stream(0) and drv.Stream(5) and drv.Stream(0) == 0
     assert repr(drv.Stream(0)) == "<Default HIP stream>"
     assert int(drv.Stream(9)) == 9 and drv.Stream(9).__cuda_stream__() == (0, 9)
 

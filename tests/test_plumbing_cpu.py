@@ -5,10 +5,13 @@ import numpy as np
 import pytest
 
 import numba_cuda_amd as cuda
-from tests import ndarray_cases, plumbing_cases
+from tests import host_stream_cases, memory_cases, ndarray_cases, plumbing_cases, slicing_cases
+
+CASES = (plumbing_cases.ALL + ndarray_cases.ALL + slicing_cases.ALL + memory_cases.ALL
+         + host_stream_cases.ALL)
 
 
-@pytest.mark.parametrize("case", plumbing_cases.ALL + ndarray_cases.ALL, ids=lambda f: f.__name__)
+@pytest.mark.parametrize("case", CASES, ids=lambda f: f.__name__)
 def test_plumbing(case, fake_gpu):
     case(cuda)
 
