@@ -178,7 +178,11 @@ class DeviceNDArrayBase:
         return self.gpu_data
 
     def get_ipc_handle(self):
-        raise NotImplementedError("IPC handles are not part of this build")
+        """An IpcArrayHandle built from whatever the context's memory manager returns
+        for this allocation (the built-in manager has no IPC support)."""
+        handle = devices.get_context().get_ipc_handle(self.gpu_data)
+        return IpcArrayHandle(ipc_handle=handle, array_desc=dict(shape=self.shape, strides=self.strides,
+                                                                 dtype=self.dtype))
 
     def _default_stream(self, stream):
         return stream if stream else self.stream
@@ -463,6 +467,29 @@ class DeviceNDArray(DeviceNDArrayBase):
         self.setitem(key, value)
 
     _do_setitem = setitem
+
+
+class IpcArrayHandle:
+    """What get_ipc_handle() returns: the memory manager's handle plus the array
+    layout; open() in another process yields a DeviceNDArray over the shared memory
+    (reference :793-835)."""
+
+    def __init__(self, ipc_handle, array_desc):
+        self._array_desc = array_desc
+        self._ipc_handle = ipc_handle
+
+    def open(self):
+        shared = self._ipc_handle.open(devices.get_context())
+        return DeviceNDArray(gpu_data=shared, **self._array_desc)
+
+    def close(self):
+        self._ipc_handle.close()
+
+    def __enter__(self):
+        return self.open()
+
+    def __exit__(self, exc_type, exc, tb):
+        self.close()
 
 
 class _HostVisibleArray(DeviceNDArrayBase, np.ndarray):

@@ -80,7 +80,7 @@ class _Runtime:
         device 0 when the thread has not chosen yet), made current."""
         if devnum is None:
             ctx = getattr(self._tls, "ctx", None)
-            if ctx is not None:          # the common case: this thread already has a device
+            if ctx is not None and ctx.prepared:   # the common case: this thread already has a device
                 return ctx
             devnum = self.current_device
             if devnum is None:

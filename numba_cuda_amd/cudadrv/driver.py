@@ -494,6 +494,16 @@ class Context:
         self.extras = {}
         self._scratch = {}   # stream handle -> device scratch for nbh_reduce
 
+    @property
+    def memory_manager(self):
+        return self._memory_manager
+
+    @memory_manager.setter
+    def memory_manager(self, manager):
+        # a manager put in by hand is initialised the next time the context is fetched
+        self._memory_manager = manager
+        self.prepared = False
+
     def reset(self):
         _logger.info("reset context of device %s", self.device.id)
         self._scratch.clear()
@@ -502,6 +512,10 @@ class Context:
 
     def prepare_for_use(self):
         self.memory_manager.initialize()
+        self.prepared = True
+
+    def get_ipc_handle(self, memory):
+        return self.memory_manager.get_ipc_handle(memory)
 
     def get_memory_info(self):
         return self.memory_manager.get_memory_info()

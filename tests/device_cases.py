@@ -1,0 +1,76 @@
+"""Device selection, reset and the gpus list as the reference's suite pins them
+(numba_cuda/numba/cuda/tests/cudadrv/test_select_device.py, test_reset_device.py,
+test_context_stack.py, test_cuda_auto_context.py), restated with the lines each case
+follows; what needs a second GPU or CUDA's context stack has no counterpart.  Run on
+the fake library and on the GPU."""
+import numbers
+import threading
+from queue import Queue
+
+import numpy as np
+
+from numba_cuda_amd.cudadrv import driver
+
+
+def _in_threads(body, count):
+    errors = Queue()
+
+    def runner():
+        try:
+            body()
+        except Exception as e:      # noqa: BLE001 - reported to the caller
+            errors.put(e)
+
+    for _ in range(count):
+        t = threading.Thread(target=runner)
+        t.start()
+        t.join()
+    found = []
+    while not errors.empty():
+        found.append(errors.get())
+    assert found == []
+
+
+def select_device_in_fresh_threads(cuda):
+    # test_select_device.py:9-36
+    def body():
+        cuda.select_device(0)
+        st = cuda.stream()
+        d = cuda.to_device(np.arange(100), stream=st)
+        st.synchronize()
+        del d
+        del st
+        cuda.synchronize()
+
+    _in_threads(body, 10)
+
+
+def select_and_close_repeatedly(cuda):
+    # test_reset_device.py:10-33
+    def body():
+        for _ in range(2):
+            for d in range(driver.driver.get_device_count()):
+                cuda.select_device(d)
+                cuda.close()
+
+    _in_threads(body, 1)
+    cuda.select_device(0)
+
+
+def gpus_list_and_memory_info(cuda):
+    # test_context_stack.py:11-44, test_cuda_auto_context.py:8-19
+    assert len(cuda.gpus) > 0 and len(list(cuda.gpus)) > 0
+    for dev in cuda.list_devices():
+        with cuda.gpus[dev.id]:
+            assert cuda.gpus.current.id == dev.id
+    mem = cuda.current_context().get_memory_info()
+    assert isinstance(mem.free, numbers.Number) and mem.free == mem[0]
+    assert isinstance(mem.total, numbers.Number) and mem.total == mem[1]
+    assert mem.free <= mem.total
+    a = np.arange(10, dtype=np.float32)
+    back = np.empty_like(a)
+    cuda.to_device(a).copy_to_host(back)
+    assert np.allclose(a, back)
+
+
+ALL = [select_device_in_fresh_threads, select_and_close_repeatedly, gpus_list_and_memory_info]
