@@ -37,12 +37,14 @@ enum nbh_dtype {
     NBH_I8 = 0, NBH_I16 = 1, NBH_I32 = 2, NBH_I64 = 3,
     NBH_U8 = 4, NBH_U16 = 5, NBH_U32 = 6, NBH_U64 = 7,
     NBH_F32 = 8, NBH_F64 = 9,
-    NBH_DTYPE_COUNT = 10
+    NBH_C64 = 10, NBH_C128 = 11,   /* complex: pairs (re, im) of float32 / float64; ADD and MUL only */
+    NBH_DTYPE_COUNT = 12
 };
 
 /* binary operators understood by nbh_reduce.  Semantics are those the reference's
  * JIT gives the Python functor (cpython/builtins.py:224-269):
- *   ADD a + b, MUL a * b      native arithmetic, integers wrap modulo 2^bits
+ *   ADD a + b, MUL a * b      native arithmetic, integers wrap modulo 2^bits; complex
+ *                             products are (ac - bd) + (ad + bc)i, each operation rounded
  *   MAX b if b > a else a,  MIN b if b < a else a */
 enum nbh_op { NBH_ADD = 0, NBH_MUL = 1, NBH_MAX = 2, NBH_MIN = 3, NBH_OP_COUNT = 4 };
 

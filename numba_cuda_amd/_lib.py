@@ -70,7 +70,7 @@ SIGNATURES = {
 # enum nbh_dtype / enum nbh_op
 DTYPE_CODES = {"int8": 0, "int16": 1, "int32": 2, "int64": 3,
                "uint8": 4, "uint16": 5, "uint32": 6, "uint64": 7,
-               "float32": 8, "float64": 9}
+               "float32": 8, "float64": 9, "complex64": 10, "complex128": 11}
 OP_CODES = {"add": 0, "mul": 1, "max": 2, "min": 3}
 
 # hipError_t values the Python layer branches on

@@ -43,6 +43,26 @@ constexpr size_t kScratchBytes = kHeaderBytes + sizeof(uint64_t) * kMaxGrid;
 constexpr int kGridPerCU = 2;
 constexpr int kUnroll = 4;
 
+// ---- complex elements -------------------------------------------------------------
+// An aggregate (it lives in unions with raw packets).  Multiplication is the plain
+// formula (ac - bd) + (ad + bc)i, four products and two sums each rounded once, which
+// is what the reference's JIT emits for `a * b` on complex operands.
+template <typename R> struct Cplx {
+    R re, im;
+};
+template <typename R> __device__ __forceinline__ Cplx<R> operator+(Cplx<R> a, Cplx<R> b)
+{
+    return {a.re + b.re, a.im + b.im};
+}
+template <typename R> __device__ __forceinline__ Cplx<R> operator*(Cplx<R> a, Cplx<R> b)
+{
+    return {a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+}
+template <typename T> struct IsCplx : std::false_type {};
+template <typename R> struct IsCplx<Cplx<R>> : std::true_type {};
+// real or complex floating point: the accumulator is the element type itself
+template <typename T> struct IsInexact : std::integral_constant<bool, std::is_floating_point<T>::value || IsCplx<T>::value> {};
+
 // ---- operators -----------------------------------------------------------------
 struct OpAdd {
     template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a + b; }
@@ -66,13 +86,15 @@ template <typename T, typename Op> struct AccOf {
     using wide_int = typename std::conditional<
         sizeof(T) == 8, typename std::conditional<arith || std::is_unsigned<T>::value, uint64_t, int64_t>::type,
         typename std::conditional<arith || std::is_unsigned<T>::value, uint32_t, int32_t>::type>::type;
-    using type = typename std::conditional<std::is_floating_point<T>::value, T, wide_int>::type;
+    using type = typename std::conditional<IsInexact<T>::value, T, wide_int>::type;
 };
 
 template <typename T, typename Op> __device__ __forceinline__ typename AccOf<T, Op>::type identity_of()
 {
     using A = typename AccOf<T, Op>::type;
-    if constexpr (std::is_same<Op, OpAdd>::value)
+    if constexpr (IsCplx<T>::value)
+        return A{std::is_same<Op, OpMul>::value ? 1 : 0, 0};
+    else if constexpr (std::is_same<Op, OpAdd>::value)
         return A(0);
     else if constexpr (std::is_same<Op, OpMul>::value)
         return A(1);
@@ -95,11 +117,18 @@ template <typename A, int CTRL> __device__ __forceinline__ A dpp(A v)
     if constexpr (sizeof(A) == 4) {
         uint32_t b = __builtin_bit_cast(uint32_t, v);
         return __builtin_bit_cast(A, dpp_move<CTRL>(b));
-    } else {
+    } else if constexpr (sizeof(A) == 8) {
         uint64_t b = __builtin_bit_cast(uint64_t, v);
         uint32_t lo = dpp_move<CTRL>((uint32_t)b);
         uint32_t hi = dpp_move<CTRL>((uint32_t)(b >> 32));
         return __builtin_bit_cast(A, ((uint64_t)hi << 32) | lo);
+    } else {
+        static_assert(sizeof(A) == 16, "accumulators are 4, 8 or 16 bytes");
+        nbh_u32x4 b = __builtin_bit_cast(nbh_u32x4, v);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            b[k] = dpp_move<CTRL>(b[k]);
+        return __builtin_bit_cast(A, b);
     }
 }
 
@@ -108,11 +137,17 @@ template <typename A> __device__ __forceinline__ A read_lane(A v, int lane)
     if constexpr (sizeof(A) == 4) {
         uint32_t b = __builtin_bit_cast(uint32_t, v);
         return __builtin_bit_cast(A, (uint32_t)__builtin_amdgcn_readlane((int)b, lane));
-    } else {
+    } else if constexpr (sizeof(A) == 8) {
         uint64_t b = __builtin_bit_cast(uint64_t, v);
         uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, lane);
         uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), lane);
         return __builtin_bit_cast(A, ((uint64_t)hi << 32) | lo);
+    } else {
+        nbh_u32x4 b = __builtin_bit_cast(nbh_u32x4, v);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            b[k] = (uint32_t)__builtin_amdgcn_readlane((int)b[k], lane);
+        return __builtin_bit_cast(A, b);
     }
 }
 
@@ -140,8 +175,15 @@ template <typename A, typename Op> __device__ __forceinline__ A block_fold(A v, 
                      Op::apply(Op::apply(lds[4], lds[5]), Op::apply(lds[6], lds[7])));
 }
 
-template <typename A> struct BitsOf {
-    using type = typename std::conditional<sizeof(A) == 8, uint64_t, uint32_t>::type;
+// A partial is published as kWords words of type Word (16-byte accumulators as two
+// 8-byte words; each word is one atomic store, the ticket is drawn after all of them
+// have been acknowledged).
+template <typename A> struct WordsOf {
+    using Word = typename std::conditional<sizeof(A) == 4, uint32_t, uint64_t>::type;
+    static constexpr int kWords = (int)(sizeof(A) / sizeof(Word));
+    struct Image {
+        Word w[kWords];
+    };
 };
 
 // ---- the kernel ------------------------------------------------------------------
@@ -155,9 +197,14 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
                                                         unsigned *__restrict__ ticket)
 {
     using A = typename AccOf<T, Op>::type;
-    using Bits = typename BitsOf<A>::type;
+    using Word = typename WordsOf<A>::Word;
+    using Image = typename WordsOf<A>::Image;
+    constexpr int kWords = WordsOf<A>::kWords;
     constexpr int V = 16 / (int)sizeof(T);
-    typedef T VecT __attribute__((ext_vector_type(V)));
+    union VecT {  // one 16-byte packet of V elements
+        nbh_u32x4 raw;
+        T item[V];
+    };
 
     __shared__ A lds[kWaves];
     __shared__ bool last_block;
@@ -169,7 +216,7 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
         acc[j] = identity_of<T, Op>();
 
     // contiguous slice of vectors owned by this workgroup
-    const VecT *__restrict__ vin = reinterpret_cast<const VecT *>(in + head);
+    const nbh_u32x4 *__restrict__ vin = reinterpret_cast<const nbh_u32x4 *>(in + head);
     const int64_t per = (nvec + gridDim.x - 1) / gridDim.x;
     const int64_t begin = (int64_t)blockIdx.x * per;
     int64_t end = begin + per;
@@ -195,18 +242,19 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
             VecT v[kUnroll];
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
-                v[u] = __builtin_nontemporal_load(&vin[i + u * kBlock]);
+                v[u].raw = __builtin_nontemporal_load(&vin[i + u * kBlock]);
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
                 for (int j = 0; j < V; ++j)
-                    acc[j] = Op::apply(acc[j], (A)v[u][j]);
+                    acc[j] = Op::apply(acc[j], (A)v[u].item[j]);
         }
         for (; i < end; i += kBlock) {
-            VecT v = __builtin_nontemporal_load(&vin[i]);
+            VecT v;
+            v.raw = __builtin_nontemporal_load(&vin[i]);
 #pragma unroll
             for (int j = 0; j < V; ++j)
-                acc[j] = Op::apply(acc[j], (A)v[j]);
+                acc[j] = Op::apply(acc[j], (A)v.item[j]);
         }
 
         // elements outside the aligned body: fewer than 2 V, one per lane of workgroup 0
@@ -231,10 +279,13 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
         return;
     }
 
-    Bits *partials = reinterpret_cast<Bits *>(partials_raw);
+    Word *partials = reinterpret_cast<Word *>(partials_raw);
     if (tid == 0) {
-        __hip_atomic_store(&partials[blockIdx.x], __builtin_bit_cast(Bits, total), __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+        const Image img = __builtin_bit_cast(Image, total);
+#pragma unroll
+        for (int w = 0; w < kWords; ++w)
+            __hip_atomic_store(&partials[(int64_t)blockIdx.x * kWords + w], img.w[w], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
         // wait for the write-through store to be acknowledged before the ticket is drawn
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -248,8 +299,12 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
 
     A fin = identity_of<T, Op>();
     for (int k = tid; k < (int)gridDim.x; k += kBlock) {
-        Bits b = __hip_atomic_load(&partials[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        fin = Op::apply(fin, __builtin_bit_cast(A, b));
+        Image img;
+#pragma unroll
+        for (int w = 0; w < kWords; ++w)
+            img.w[w] = __hip_atomic_load(&partials[(int64_t)k * kWords + w], __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+        fin = Op::apply(fin, __builtin_bit_cast(A, img));
     }
     fin = block_fold<A, Op>(fin, lds);
     if (tid == 0) {
@@ -279,8 +334,9 @@ int launch(const void *in, int64_t n, int64_t stride, const void *init, void *ou
     const int64_t per_block = (int64_t)kBlock * kUnroll;
     int64_t grid = (units + per_block - 1) / per_block;
     int64_t cap = (int64_t)nbh_cu_count() * kGridPerCU;
-    if (cap > kMaxGrid)
-        cap = kMaxGrid;
+    constexpr int64_t kSlots = (int64_t)kMaxGrid * 8 / (sizeof(T) > 8 ? 16 : 8);  // partials that fit the scratch
+    if (cap > kSlots)
+        cap = kSlots;
     if (grid > cap)
         grid = cap;
     if (grid < 1)
@@ -312,6 +368,18 @@ int launch_op(int op, const void *in, int64_t n, int64_t stride, const void *ini
     }
 }
 
+// complex elements: sums and products only (there is no order to take a maximum by)
+template <typename T>
+int launch_op_complex(int op, const void *in, int64_t n, int64_t stride, const void *init, void *out,
+                      void *scratch, hipStream_t s)
+{
+    switch (op) {
+    case NBH_ADD: return launch<T, OpAdd>(in, n, stride, init, out, scratch, s);
+    case NBH_MUL: return launch<T, OpMul>(in, n, stride, init, out, scratch, s);
+    default: return (int)hipErrorInvalidValue;
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -336,6 +404,8 @@ int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, 
     case NBH_U64: return launch_op<uint64_t>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_F32: return launch_op<float>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_F64: return launch_op<double>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_C64: return launch_op_complex<Cplx<float>>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_C128: return launch_op_complex<Cplx<double>>(op, in, n, in_stride, init, out, scratch, s);
     default: return (int)hipErrorInvalidValue;
     }
 }

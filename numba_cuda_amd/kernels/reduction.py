@@ -158,6 +158,16 @@ class Reduce:
             except TypeError:
                 pass
         self._opcode = _lib.OP_CODES[self._op]
+        self._codes = {}    # dtype -> element code, filled once the pairing with the operator is checked
+
+    def _element_code(self, dtype):
+        code = _DTYPE_CODE.get(dtype)
+        if code is None:
+            raise NotImplementedError("Reduce does not support dtype %s" % dtype)
+        if dtype.kind == "c" and self._op in ("max", "min"):
+            # the reference fails the same way, at compile time: complex numbers are not ordered
+            raise TypeError("max / min are not defined for %s" % dtype)
+        return code
 
     def __call__(self, arr, size=None, res=None, init=0, stream=0):
         """Full reduction of `arr`.
@@ -178,9 +188,9 @@ class Reduce:
         if arr.size < 1:
             return dtype.type(init)          # `res` is left untouched, as in the reference
 
-        code = _DTYPE_CODE.get(dtype)
+        code = self._codes.get(dtype)
         if code is None:
-            raise NotImplementedError("Reduce does not support dtype %s" % dtype)
+            code = self._codes[dtype] = self._element_code(dtype)
 
         ctx = devices.get_context()
         if not _driver.is_device_memory(arr):

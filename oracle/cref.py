@@ -22,7 +22,10 @@ SUFFIX = {
     "u8": np.uint8, "u16": np.uint16, "u32": np.uint32, "u64": np.uint64,
     "f32": np.float32, "f64": np.float64,
 }
-_SUFFIX_OF = {np.dtype(v): k for k, v in SUFFIX.items()}
+# complex elements reduce with add and mul only
+COMPLEX_SUFFIX = {"c64": np.complex64, "c128": np.complex128}
+COMPLEX_OPS = ("add", "mul")
+_SUFFIX_OF = {np.dtype(v): k for k, v in list(SUFFIX.items()) + list(COMPLEX_SUFFIX.items())}
 OPS = ("add", "mul", "max", "min")
 
 STATE_DTYPE = np.dtype([("s0", np.uint64), ("s1", np.uint64)], align=True)
@@ -56,6 +59,10 @@ def lib():
             getattr(L, "orc_xoro_fill_" + kind).argtypes = [_vp, _c_i64, _vp, _c_i64]
         for op in OPS:
             for sfx in SUFFIX:
+                for fam in ("fold", "tree"):
+                    getattr(L, f"orc_{fam}_{op}_{sfx}").argtypes = [_vp, _c_i64, _vp, _vp]
+        for op in COMPLEX_OPS:
+            for sfx in COMPLEX_SUFFIX:
                 for fam in ("fold", "tree"):
                     getattr(L, f"orc_{fam}_{op}_{sfx}").argtypes = [_vp, _c_i64, _vp, _vp]
         L.orc_sum_exact_f32.argtypes = [_vp, _c_i64, _vp, _vp]

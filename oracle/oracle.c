@@ -315,6 +315,34 @@ DEFINE_REDUCE_INT(u64, uint64_t, uint64_t)
 DEFINE_REDUCE_FLT(f32, float)
 DEFINE_REDUCE_FLT(f64, double)
 
+/* Complex elements: `a + b` componentwise, `a * b` by the plain formula
+ * (ac - bd) + (ad + bc)i with every product and sum rounded once - what the
+ * reference's JIT emits for complex operands (no special-value recovery, no fused
+ * operations in this restatement; the compiled reference may contract to FMA, which
+ * is why complex PRODUCTS are compared with a tolerance).  No max / min. */
+typedef struct { float re, im; } orc_c64;
+typedef struct { double re, im; } orc_c128;
+static inline orc_c64 c64_add(orc_c64 a, orc_c64 b) { orc_c64 r = {a.re + b.re, a.im + b.im}; return r; }
+static inline orc_c128 c128_add(orc_c128 a, orc_c128 b) { orc_c128 r = {a.re + b.re, a.im + b.im}; return r; }
+static inline orc_c64 c64_mul(orc_c64 a, orc_c64 b)
+{
+    orc_c64 r = {a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+    return r;
+}
+static inline orc_c128 c128_mul(orc_c128 a, orc_c128 b)
+{
+    orc_c128 r = {a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+    return r;
+}
+#define OP_ADD_C64(T, U, a, b) c64_add(a, b)
+#define OP_MUL_C64(T, U, a, b) c64_mul(a, b)
+#define OP_ADD_C128(T, U, a, b) c128_add(a, b)
+#define OP_MUL_C128(T, U, a, b) c128_mul(a, b)
+DEFINE_REDUCE(add_c64, orc_c64, orc_c64, OP_ADD_C64)
+DEFINE_REDUCE(mul_c64, orc_c64, orc_c64, OP_MUL_C64)
+DEFINE_REDUCE(add_c128, orc_c128, orc_c128, OP_ADD_C128)
+DEFINE_REDUCE(mul_c128, orc_c128, orc_c128, OP_MUL_C128)
+
 /* Association-free yardsticks for the floating-point tolerance
  * |err| <= 2 n eps sum|x|: the sum and the sum of magnitudes accumulated in
  * long double with Neumaier compensation. */

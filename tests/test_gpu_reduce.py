@@ -111,6 +111,63 @@ def test_every_operator_and_dtype_against_oracle(op, sfx):
             assert got == cref.tree(op, a, init)
 
 
+@pytest.mark.parametrize("dtype", [np.complex64, np.complex128])
+def test_complex_sums_and_products(dtype):
+    """Complex elements: sums within 2 n eps sum|x| per component of the exact sums;
+    products of near-unit factors within 8 n eps (relative) of the oracle's value in
+    the reference's association order; integers-valued inputs exactly."""
+    dt = np.dtype(dtype)
+    real = np.float32 if dt == np.complex64 else np.float64
+    eps = np.finfo(real).eps
+    rng = np.random.default_rng(21)
+    add, mul = cuda.Reduce(lambda a, b: a + b), cuda.Reduce(lambda a, b: a * b)
+    for n in (1, 2, 3, 63, 64, 65, 1000, 4097, 300001, 2**21 + 5):
+        _say("complex reduce", dt, n)
+        a = (rng.standard_normal(n) + 1j * rng.standard_normal(n)).astype(dt)
+        got = add(a, init=1 - 2j)
+        assert got.dtype == dt
+        for part, off in (("real", 1.0), ("imag", -2.0)):
+            exact, sum_abs = cref.sum_exact(np.ascontiguousarray(getattr(a, part)))
+            tol = 2 * n * eps * (sum_abs + 2.0)                       # tolerance: 2 n eps sum|x|
+            assert abs(float(getattr(got, part)) - (exact + off)) <= tol
+        # exactly representable partial sums: every association gives the same bits
+        k = (rng.integers(-1000, 1000, n) + 1j * rng.integers(-1000, 1000, n)).astype(dt)
+        assert add(k, init=3 + 4j) == cref.tree("add", k, 3 + 4j) == cref.fold("add", k, 3 + 4j)
+        m = min(n, 5000)
+        u = (np.exp(1j * rng.uniform(0, 2 * np.pi, m)) * (1 + 1e-3 * rng.standard_normal(m))).astype(dt)
+        got = mul(u, init=1)
+        want = cref.tree("mul", u, 1)
+        assert abs(got - want) <= 8 * m * eps * abs(want)             # tolerance: 8 n eps, relative
+    # Gaussian integers: products are exact while they fit the mantissa
+    g = np.array([1 + 1j, 2 - 1j, -1 + 3j, 2 + 2j, 1 - 4j, 3 + 1j], dtype=dt)
+    assert mul(g, init=1j) == np.prod(g.astype(np.complex128)) * 1j == cref.tree("mul", g, 1j)
+    d = cuda.to_device((rng.standard_normal(1001) + 1j * rng.standard_normal(1001)).astype(dt))
+    np.testing.assert_allclose(add(d[::-2]), d.copy_to_host()[::-2].sum(), rtol=1e-4 if dt == np.complex64 else 1e-12)
+    res = cuda.device_array(1, dt)
+    assert add(d, res=res) is None and res.copy_to_host()[0] == add(d)
+    for op in (lambda a, b: max(a, b), lambda a, b: min(a, b)):
+        with pytest.raises(TypeError, match="not defined for complex"):
+            cuda.Reduce(op)(d)
+
+
+def test_simulator_case_65536_uniform_seed_0():
+    """The CPU-runnable configuration of the reference (its simulator: a strict left
+    fold of 65 536 float32 drawn uniform [-1, 1) from seed 0, init 0) beside the GPU:
+    both within 2 n eps sum|x| of the exact sum, hence within twice that of each other."""
+    from oracle import sim
+    a = np.random.default_rng(0).uniform(-1, 1, 65536).astype(np.float32)
+    want = sim.Reduce(lambda x, y: x + y)(a, init=0)
+    assert isinstance(want, np.float32) and want == cref.fold("add", a, 0)
+    got = sum_reduce(cuda.to_device(a), init=0)
+    assert got.dtype == np.float32
+    exact, sum_abs = cref.sum_exact(a)
+    tol = 2 * a.size * np.finfo(np.float32).eps * sum_abs          # tolerance: 2 n eps sum|x|
+    assert abs(float(got) - exact) <= tol and abs(float(want) - exact) <= tol
+    assert abs(float(got) - float(want)) <= 2 * tol
+    res = cuda.device_array(1, np.float32)
+    assert sum_reduce(a, res=res, init=0) is None and res.copy_to_host()[0] == got
+
+
 def test_runs_are_bitwise_reproducible():
     rng = np.random.default_rng(5)
     a = cuda.to_device(rng.standard_normal(3_000_017).astype(np.float32))

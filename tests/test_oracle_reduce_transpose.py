@@ -148,6 +148,27 @@ def test_minmax_follow_python_semantics_for_nan_and_signed_zero():
     assert math.copysign(1, cref.fold("min", z, 0.0)) == 1.0
 
 
+def test_complex_reductions_of_the_oracle():
+    """Pins: componentwise sums equal the real-valued oracle on each component (same
+    association); products of Gaussian integers are exact and equal NumPy's; a
+    conjugated input gives the conjugated product (sign symmetry of the formula)."""
+    rng = np.random.default_rng(4)
+    for dt, real in ((np.complex64, np.float32), (np.complex128, np.float64)):
+        for n in (1, 31, 32, 33, 127, 128, 129, 8192, 8321, 20000):
+            a = (rng.standard_normal(n) + 1j * rng.standard_normal(n)).astype(dt)
+            for fam in (cref.fold, cref.tree):
+                got = fam("add", a, 0.5 - 0.25j)
+                re = fam("add", np.ascontiguousarray(a.real), real(0.5))
+                im = fam("add", np.ascontiguousarray(a.imag), real(-0.25))
+                assert (got.real, got.imag) == (re, im)
+        g = (rng.integers(-3, 4, 12) + 1j * rng.integers(-3, 4, 12)).astype(dt)
+        want = np.prod(g.astype(np.complex128))
+        assert cref.fold("mul", g, 1) == want == cref.tree("mul", g, 1)
+        u = np.exp(1j * rng.uniform(0, 6, 300)).astype(dt)
+        assert cref.tree("mul", np.conj(u), 1) == np.conj(cref.tree("mul", u, 1))
+        assert abs(abs(cref.tree("mul", u, 1)) - 1) < 300 * 4 * np.finfo(real).eps
+
+
 def test_fold_matches_simulator_path():
     rng = np.random.default_rng(0)
     a = rng.uniform(-1, 1, 65536).astype(np.float32)       # the 65536-element simulator case
