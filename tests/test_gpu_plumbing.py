@@ -88,6 +88,42 @@ def test_flat_assignment_at_every_alignment(dtype):
             assert got.tobytes() == want.tobytes(), (n, d_off, s_off)
 
 
+def test_large_pageable_copies_go_through_the_staging_ring():
+    """Host copies of 32 MiB and more without a stream are pipelined through page-locked
+    buffers by several threads: ragged sizes, odd offsets, fresh destination pages,
+    two Python threads at once, and the ordering hipMemcpy gives after work on a stream."""
+    import threading
+    rng = np.random.default_rng(14)
+    big = rng.integers(0, 255, (80 << 20) + 12345, dtype=np.uint8)
+    for lo, n in ((0, big.size), (1, (32 << 20)), (4097, (48 << 20) + 1), (3, (32 << 20) - 1)):
+        src = big[lo:lo + n]
+        d = cuda.to_device(src)                                  # pageable -> device
+        back = d.copy_to_host()                                  # device -> fresh pageable memory
+        assert back.tobytes() == src.tobytes(), (lo, n)
+        into = np.zeros(n + 10, np.uint8)
+        d.copy_to_host(into[5:5 + n])                            # into the middle of an existing array
+        assert into[5:5 + n].tobytes() == src.tobytes() and not into[:5].any() and not into[-5:].any()
+    # ordering: a kernel on a (blocking) stream, then a synchronous copy without any wait in between
+    st = cuda.stream()
+    a = cuda.to_device(big[: 64 << 20])
+    b = cuda.device_array(64 << 20, np.uint8)
+    b.setitem(slice(None), a, stream=st)
+    assert b.copy_to_host().tobytes() == big[: 64 << 20].tobytes()
+    # two threads copying at the same time
+    results = {}
+
+    def worker(key, lo):
+        dd = cuda.to_device(big[lo:lo + (40 << 20)])
+        results[key] = dd.copy_to_host().tobytes() == big[lo:lo + (40 << 20)].tobytes()
+
+    threads = [threading.Thread(target=worker, args=(k, k * 1000 + 7)) for k in range(3)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert results == {0: True, 1: True, 2: True}
+
+
 def test_large_device_to_device_copies():
     """copy_to_device between device arrays of a MiB and more runs on the library's own
     copy kernel (smaller ones on hipMemcpy): with and without a stream, at odd offsets."""
