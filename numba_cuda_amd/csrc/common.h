@@ -22,11 +22,11 @@ static inline hipStream_t nbh_hip_stream(nbh_stream_t s) { return (hipStream_t)s
 // Number of compute units of the current device (cached per device).
 int nbh_cu_count();
 
-// Large synchronous copies between pageable host memory and the device through a
+// Large copies between pageable host memory and the device through a
 // ring of page-locked buffers and a few copy threads (hostcopy.hip).  0: done;
 // -1: not a case for the pipeline, use hipMemcpy; otherwise a hipError_t.
-int nbh_staged_d2h(void *dst, const void *src, size_t nbytes);
-int nbh_staged_h2d(void *dst, const void *src, size_t nbytes);
+int nbh_staged_d2h(void *dst, const void *src, size_t nbytes, hipStream_t stream);
+int nbh_staged_h2d(void *dst, const void *src, size_t nbytes, hipStream_t stream);
 
 // dst[0:nbytes] = src[0:nbytes] with the flat copy kernel of nbh_assign, on `stream`
 // (asynchronous).  Both ranges must be memory the current device can address.

@@ -12,10 +12,11 @@
 // pipeline off).  Result, same box: host-to-device 53 GB/s, device-to-host 50 GB/s,
 // also into untouched memory.
 //
-// Ordering is hipMemcpy's: the DMA legs are issued on the legacy default stream, so
-// they wait for earlier work of every blocking stream, and the call returns when the
-// whole copy is done.  One pipelined copy runs at a time per process; a second
-// caller waits for the first.
+// Ordering is hipMemcpy's / hipMemcpyAsync's: the DMA legs are issued on the stream the
+// caller names (the legacy default stream when none is named, so that they wait for
+// earlier work of every blocking stream), and the call returns when the whole copy is
+// done - as HIP's own asynchronous copies of pageable memory do.  One pipelined copy
+// runs at a time per process; a second caller waits for the first.
 #include "common.h"
 
 #include <algorithm>
@@ -171,7 +172,7 @@ bool pageable(const void *host)
 // for the pipeline (too small, page-locked host memory, switched off): the caller
 // then uses hipMemcpy.
 
-int nbh_staged_d2h(void *dst, const void *src, size_t nbytes)
+int nbh_staged_d2h(void *dst, const void *src, size_t nbytes, hipStream_t stream)
 {
     if (nbytes < kMinBytes || !pageable(dst))
         return -1;
@@ -187,8 +188,8 @@ int nbh_staged_d2h(void *dst, const void *src, size_t nbytes)
     auto span = [&](size_t i) { return std::min(kChunk, nbytes - i * kChunk); };
     auto fetch = [&](size_t i) -> int {  // device -> staging buffer i % kRing
         const int k = (int)(i % kRing);
-        NBH_TRY(hipMemcpyAsync(ring->buf[k], (const char *)src + i * kChunk, span(i), hipMemcpyDeviceToHost, 0));
-        NBH_TRY(hipEventRecord(ring->landed[k], 0));
+        NBH_TRY(hipMemcpyAsync(ring->buf[k], (const char *)src + i * kChunk, span(i), hipMemcpyDeviceToHost, stream));
+        NBH_TRY(hipEventRecord(ring->landed[k], stream));
         return 0;
     };
     for (size_t i = 0; i < std::min<size_t>(kRing, chunks); ++i)
@@ -204,7 +205,7 @@ int nbh_staged_d2h(void *dst, const void *src, size_t nbytes)
     return 0;
 }
 
-int nbh_staged_h2d(void *dst, const void *src, size_t nbytes)
+int nbh_staged_h2d(void *dst, const void *src, size_t nbytes, hipStream_t stream)
 {
     if (nbytes < kMinBytes || !pageable(src))
         return -1;
@@ -223,8 +224,8 @@ int nbh_staged_h2d(void *dst, const void *src, size_t nbytes)
         if (i >= (size_t)kRing)  // the DMA that read this buffer kRing chunks ago must be over
             NBH_TRY(hipEventSynchronize(ring->landed[k]));
         p.crew->copy(ring->buf[k], (const char *)src + i * kChunk, n);
-        NBH_TRY(hipMemcpyAsync((char *)dst + i * kChunk, ring->buf[k], n, hipMemcpyHostToDevice, 0));
-        NBH_TRY(hipEventRecord(ring->landed[k], 0));
+        NBH_TRY(hipMemcpyAsync((char *)dst + i * kChunk, ring->buf[k], n, hipMemcpyHostToDevice, stream));
+        NBH_TRY(hipEventRecord(ring->landed[k], stream));
     }
-    return (int)hipStreamSynchronize(0);
+    return (int)hipStreamSynchronize(stream);
 }

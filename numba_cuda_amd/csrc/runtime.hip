@@ -159,24 +159,21 @@ static int copy(void *dst, const void *src, size_t nbytes, hipMemcpyKind kind, n
         return (int)hipMemcpyAsync(dst, src, nbytes, kind, nbh_hip_stream(stream));
     return (int)hipMemcpy(dst, src, nbytes, kind);
 }
-// Without a stream the call returns when the copy is done, so large copies of
-// pageable memory can be pipelined through page-locked buffers by the library itself.
+// Large copies of pageable memory are pipelined through page-locked buffers by the
+// library itself (with or without a stream: a copy of pageable memory cannot outlive
+// the call either way).
 int nbh_memcpy_h2d(void *dst, const void *src, size_t nbytes, nbh_stream_t stream)
 {
-    if (!stream) {
-        const int rc = nbh_staged_h2d(dst, src, nbytes);
-        if (rc >= 0)
-            return rc;
-    }
+    const int rc = nbh_staged_h2d(dst, src, nbytes, nbh_hip_stream(stream));
+    if (rc >= 0)
+        return rc;
     return copy(dst, src, nbytes, hipMemcpyHostToDevice, stream);
 }
 int nbh_memcpy_d2h(void *dst, const void *src, size_t nbytes, nbh_stream_t stream)
 {
-    if (!stream) {
-        const int rc = nbh_staged_d2h(dst, src, nbytes);
-        if (rc >= 0)
-            return rc;
-    }
+    const int rc = nbh_staged_d2h(dst, src, nbytes, nbh_hip_stream(stream));
+    if (rc >= 0)
+        return rc;
     return copy(dst, src, nbytes, hipMemcpyDeviceToHost, stream);
 }
 // Plain device memory of the current device?  (Not host-mapped or managed memory,

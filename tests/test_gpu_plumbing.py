@@ -109,6 +109,11 @@ def test_large_pageable_copies_go_through_the_staging_ring():
     b = cuda.device_array(64 << 20, np.uint8)
     b.setitem(slice(None), a, stream=st)
     assert b.copy_to_host().tobytes() == big[: 64 << 20].tobytes()
+    # on a stream: the legs run on that stream, the call still returns a finished copy
+    d = cuda.to_device(big[: 50 << 20], stream=st)
+    got = np.empty(50 << 20, np.uint8)
+    d.copy_to_host(got, stream=st)
+    assert got.tobytes() == big[: 50 << 20].tobytes()
     # two threads copying at the same time
     results = {}
 
