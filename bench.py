@@ -193,7 +193,7 @@ def _workload(name, cuda):
                 nrandom.init_xoroshiro128p_states(states, 42, 0, stream)
             return dict(desc="create_xoroshiro128p_states 2^24 states, seed 42", dtype="u64",
                         algo_bytes=16 * n, units=n, step=step, stream=stream, host=None,
-                        kernel="init_states_kernel", keep=(states,))
+                        kernel="init_states_tables_kernel", keep=(states,))
         if name == "rng_uniform_f32":
             out = cuda.device_array(n * 64, np.float32)
 
@@ -201,7 +201,7 @@ def _workload(name, cuda):
                 nrandom.xoroshiro128p_fill(states, out, 64, nrandom.UNIFORM, stream)
             return dict(desc="xoroshiro128p 2^24 generators x 64 uniform float32", dtype="u64",
                         algo_bytes=4 * n * 64 + 32 * n, units=n * 64, step=step, stream=stream, host=None,
-                        kernel="fill_kernel", keep=(states, out))
+                        kernel="fill_kernel<UniformF32>", keep=(states, out))
         if name == "rng_normal_f64":
             out = cuda.device_array(n * 16, np.float64)
 
@@ -209,7 +209,7 @@ def _workload(name, cuda):
                 nrandom.xoroshiro128p_fill(states, out, 16, nrandom.NORMAL, stream)
             return dict(desc="xoroshiro128p 2^24 generators x 16 normal float64", dtype="f64",
                         algo_bytes=8 * n * 16 + 32 * n, units=n * 16, step=step, stream=stream, host=None,
-                        kernel="fill_kernel", keep=(states, out))
+                        kernel="fill_kernel<NormalF64>", keep=(states, out))
     if name == "copy_f32":
         # flat device-to-device assignment: the plain copy kernel of known size that
         # the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are calibrated against

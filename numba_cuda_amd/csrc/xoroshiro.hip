@@ -20,13 +20,14 @@
 // The reference's layout out[t*count + i] gives every lane its own run of `count`
 // values, so values are parked in LDS for a round and written back with the run
 // index fastest: every store instruction of a wavefront covers whole 128-byte lines.
+// The Box-Muller normals take their logarithm and cosine from boxmuller_math.h.
 //
 // HBM roofline: out bytes written + 2 * 16 bytes of state per generator.
 #include "common.h"
 #include "boxmuller_math.h"
-#include <type_traits>
 
 #include <mutex>
+#include <type_traits>
 
 namespace {
 
