@@ -82,6 +82,18 @@ int nbh_free(void *dptr);
  * from the host and the device at the same address; attach_global != 0 ->
  * attached to every stream, 0 -> host-attached.  Release with nbh_free. */
 int nbh_malloc_managed(void **ptr, size_t nbytes, int attach_global);
+/* A caching allocator behind the external-memory-manager interface
+ * (cudadrv/driver.py:592-703 BaseCUDAMemoryManager; the reference ships none and
+ * points to RMM's pool for this): nbh_pool_malloc hands out a block of the current
+ * device, nbh_pool_free takes it back WITHOUT freeing it.  A block is handed out again
+ * only after the work that had been submitted, through this library, to any stream
+ * before the free has completed (events, no host-side wait).  nbh_pool_trim returns
+ * every idle block to the driver; nbh_pool_stats reports bytes idle / handed out and
+ * how many requests were served from the pool (hits) or by hipMalloc (misses). */
+int nbh_pool_malloc(void **dptr, size_t nbytes);
+int nbh_pool_free(void *dptr);
+int nbh_pool_trim(void);
+int nbh_pool_stats(size_t *idle_bytes, size_t *live_bytes, uint64_t *hits, uint64_t *misses);
 /* cudadrv/driver.py:747-779 memhostalloc (cuMemHostAlloc / cuMemFreeHost).
  * flags: bit 0 portable, bit 1 device-mapped, bit 2 write-combined */
 int nbh_host_alloc(void **hptr, size_t nbytes, unsigned flags);

@@ -34,6 +34,10 @@ SIGNATURES = {
     "nbh_malloc": (c_int, [P(c_vp), c_size]),
     "nbh_free": (c_int, [c_vp]),
     "nbh_malloc_managed": (c_int, [P(c_vp), c_size, c_int]),
+    "nbh_pool_malloc": (c_int, [P(c_vp), c_size]),
+    "nbh_pool_free": (c_int, [c_vp]),
+    "nbh_pool_trim": (c_int, []),
+    "nbh_pool_stats": (c_int, [P(c_size), P(c_size), P(ctypes.c_uint64), P(ctypes.c_uint64)]),
     "nbh_host_alloc": (c_int, [P(c_vp), c_size, ctypes.c_uint]),
     "nbh_host_free": (c_int, [c_vp]),
     "nbh_host_register": (c_int, [c_vp, c_size, ctypes.c_uint]),

@@ -22,6 +22,11 @@ static inline hipStream_t nbh_hip_stream(nbh_stream_t s) { return (hipStream_t)s
 // Number of compute units of the current device (cached per device).
 int nbh_cu_count();
 
+// The caching pool (pool.hip) must know which streams have had work submitted: every
+// entry point that takes a stream reports it here (a no-op until the pool is in use).
+void nbh_pool_note_stream(hipStream_t stream);
+void nbh_pool_forget_stream(hipStream_t stream);
+
 // Large copies between pageable host memory and the device through a
 // ring of page-locked buffers and a few copy threads (hostcopy.hip).  0: done;
 // -1: not a case for the pipeline, use hipMemcpy; otherwise a hipError_t.

@@ -393,6 +393,7 @@ int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, 
         ((uintptr_t)scratch) % 8 != 0)
         return (int)hipErrorInvalidValue;
     hipStream_t s = nbh_hip_stream(stream);
+    nbh_pool_note_stream(s);
     switch (dtype) {
     case NBH_I8: return launch_op<int8_t>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_I16: return launch_op<int16_t>(op, in, n, in_stride, init, out, scratch, s);

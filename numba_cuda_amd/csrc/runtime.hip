@@ -155,6 +155,7 @@ static int copy(void *dst, const void *src, size_t nbytes, hipMemcpyKind kind, n
 {
     if (nbytes == 0)
         return 0;
+    nbh_pool_note_stream(nbh_hip_stream(stream));
     if (stream)
         return (int)hipMemcpyAsync(dst, src, nbytes, kind, nbh_hip_stream(stream));
     return (int)hipMemcpy(dst, src, nbytes, kind);
@@ -164,6 +165,7 @@ static int copy(void *dst, const void *src, size_t nbytes, hipMemcpyKind kind, n
 // the call either way).
 int nbh_memcpy_h2d(void *dst, const void *src, size_t nbytes, nbh_stream_t stream)
 {
+    nbh_pool_note_stream(nbh_hip_stream(stream));
     const int rc = nbh_staged_h2d(dst, src, nbytes, nbh_hip_stream(stream));
     if (rc >= 0)
         return rc;
@@ -171,6 +173,7 @@ int nbh_memcpy_h2d(void *dst, const void *src, size_t nbytes, nbh_stream_t strea
 }
 int nbh_memcpy_d2h(void *dst, const void *src, size_t nbytes, nbh_stream_t stream)
 {
+    nbh_pool_note_stream(nbh_hip_stream(stream));
     const int rc = nbh_staged_d2h(dst, src, nbytes, nbh_hip_stream(stream));
     if (rc >= 0)
         return rc;
@@ -209,6 +212,7 @@ int nbh_memset8(void *dst, int byte, size_t nbytes, nbh_stream_t stream)
 {
     if (nbytes == 0)
         return 0;
+    nbh_pool_note_stream(nbh_hip_stream(stream));
     if (stream)
         return (int)hipMemsetAsync(dst, byte, nbytes, nbh_hip_stream(stream));
     return (int)hipMemset(dst, byte, nbytes);
@@ -225,7 +229,11 @@ int nbh_stream_create(nbh_stream_t *stream)
     *stream = (nbh_stream_t)s;
     return 0;
 }
-int nbh_stream_destroy(nbh_stream_t stream) { return (int)hipStreamDestroy(nbh_hip_stream(stream)); }
+int nbh_stream_destroy(nbh_stream_t stream)
+{
+    nbh_pool_forget_stream(nbh_hip_stream(stream));
+    return (int)hipStreamDestroy(nbh_hip_stream(stream));
+}
 int nbh_stream_synchronize(nbh_stream_t stream) { return (int)hipStreamSynchronize(nbh_hip_stream(stream)); }
 int nbh_stream_query(nbh_stream_t stream) { return (int)hipStreamQuery(nbh_hip_stream(stream)); }
 

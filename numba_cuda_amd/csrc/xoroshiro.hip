@@ -542,6 +542,7 @@ int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t 
         if (rc)
             return rc;
     }
+    nbh_pool_note_stream(nbh_hip_stream(stream));
     hipLaunchKernelGGL((fill_kernel<Gen>), dim3((unsigned)grid), dim3(kFillBlock), 0, nbh_hip_stream(stream),
                        (uint64_t *)states, n, (typename Gen::value_type *)out, count, log_table);
     return nbh_launch_status();
@@ -575,6 +576,7 @@ int nbh_xoro_init_states(void *states, int64_t n, uint64_t seed, uint64_t subseq
     if (rc)
         return rc;
     hipStream_t hs = nbh_hip_stream(stream);
+    nbh_pool_note_stream(hs);
     if (n >= kTablesFrom) {
         // one workgroup of 16 wavefronts per 65536 states, lookup tables in LDS
         const int64_t per_block = (int64_t)(kTabBlock / 64) * 64 * kInitSteps;

@@ -18,6 +18,7 @@ access and `__setitem__` ever touches the device.
 
 import copy
 import ctypes
+import functools
 import math
 from ctypes import c_void_p
 from warnings import warn
@@ -115,6 +116,13 @@ def _normalise_shape(shape):
 
 # ---- the array types -------------------------------------------------------------------
 
+@functools.lru_cache(maxsize=1024)
+def _layout_of(shape, strides, itemsize):
+    """The stride calculus object for an array that starts at offset 0.  Layout objects
+    are never modified, so arrays of the same shape and strides share one."""
+    return dummyarray.Array.from_desc(0, shape, strides, itemsize)
+
+
 class DeviceNDArrayBase:
     """An n-d array in device memory."""
 
@@ -137,7 +145,7 @@ class DeviceNDArrayBase:
         self.ndim = len(shape)
         if len(strides) != self.ndim:
             raise ValueError("strides not match ndim")
-        layout = dummyarray.Array.from_desc(0, shape, strides, self.dtype.itemsize)
+        layout = _layout_of(shape, strides, self.dtype.itemsize)
         self._dummy = layout
         self.shape, self.strides, self.size = layout.shape, layout.strides, layout.size
         if self.size == 0:
@@ -516,7 +524,7 @@ class _HostVisibleArray(DeviceNDArrayBase, np.ndarray):
 
     @property
     def _dummy(self):
-        return dummyarray.Array.from_desc(0, self.shape, self.strides, self.dtype.itemsize)
+        return _layout_of(tuple(self.shape), tuple(self.strides), self.dtype.itemsize)
 
     @property
     def alloc_size(self):

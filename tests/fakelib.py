@@ -102,6 +102,49 @@ class FakeLib:
         self._log("malloc_managed", nbytes, attach_global)
         return self.nbh_malloc(out, nbytes)
 
+    # the pool keeps blocks by exact size; nothing is ever pending on the fake
+    def nbh_pool_malloc(self, out, nbytes):
+        self._log("pool_malloc", nbytes)
+        size = max((int(nbytes) + 511) & ~511, 512)
+        idle = self.__dict__.setdefault("pool_idle", {})
+        self.__dict__.setdefault("pool_hits", 0)
+        if idle.get(size):
+            addr = idle[size].pop()
+            self.pool_hits += 1
+            self._out(out, addr)
+            return 0
+        rc = self.nbh_malloc(out, size)
+        if rc == 0:
+            self.__dict__.setdefault("pool_sizes", {})[out._obj.value] = size
+        return rc
+
+    def nbh_pool_free(self, ptr):
+        addr = _addr(ptr)
+        self._log("pool_free", addr)
+        size = self.__dict__.get("pool_sizes", {}).get(addr)
+        if size is None:
+            return HIP_ERROR_INVALID_VALUE
+        self.__dict__.setdefault("pool_idle", {}).setdefault(size, []).append(addr)
+        return 0
+
+    def nbh_pool_trim(self):
+        for size, addrs in self.__dict__.get("pool_idle", {}).items():
+            for addr in addrs:
+                self.buffers.pop(addr, None)
+                self.pool_sizes.pop(addr, None)
+        self.__dict__["pool_idle"] = {}
+        return 0
+
+    def nbh_pool_stats(self, idle, live, hits, misses):
+        idle_map = self.__dict__.get("pool_idle", {})
+        idle_bytes = sum(size * len(addrs) for size, addrs in idle_map.items())
+        total = sum(self.__dict__.get("pool_sizes", {}).values())
+        self._out(idle, idle_bytes)
+        self._out(live, total - idle_bytes)
+        self._out(hits, self.__dict__.get("pool_hits", 0))
+        self._out(misses, 0)
+        return 0
+
     def nbh_free(self, ptr):
         addr = _addr(ptr)
         self._log("free", addr)

@@ -6,11 +6,12 @@ import pytest
 
 import numba_cuda_amd as cuda
 from tests import (attr_cases, cai_cases, dealloc_cases, device_cases, emm_cases, host_stream_cases,
-                   memory_cases, ndarray_cases, plumbing_cases, record_cases, slicing_cases)
+                   memory_cases, ndarray_cases, plumbing_cases, pool_cases, record_cases, slicing_cases)
 
 # plumbing_cases: this package's own; the others restate the reference's suites
 CASES = (plumbing_cases.ALL + ndarray_cases.ALL + slicing_cases.ALL + memory_cases.ALL + host_stream_cases.ALL
-         + record_cases.ALL + dealloc_cases.ALL + emm_cases.ALL + attr_cases.ALL + device_cases.ALL + cai_cases.ALL)
+         + record_cases.ALL + dealloc_cases.ALL + emm_cases.ALL + attr_cases.ALL + device_cases.ALL + cai_cases.ALL
+         + pool_cases.ALL)
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda f: f.__name__)
