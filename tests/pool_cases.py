@@ -65,10 +65,55 @@ def pooled_arrays_reuse_blocks(cuda):
         cuda.current_context()
 
 
+def a_block_in_use_on_another_stream_is_not_handed_out(cuda):
+    """A released block that a queued kernel still reads must wait in the pool: release
+    a 256 MiB array right after starting a reduction of it on stream A, then allocate and
+    overwrite an array of the same size on stream B.  The reduction must see the old
+    contents; only after A has finished may the block come back."""
+    if _is_fake():
+        return
+    ctx = cuda.current_context()
+    ctx.reset()
+    original = ctx.memory_manager
+    ctx.memory_manager = PoolMemoryManager(context=ctx)
+    try:
+        mgr = cuda.current_context().memory_manager
+        n = 1 << 26
+        sa, sb = cuda.stream(), cuda.stream()
+        res = cuda.device_array(1, np.int32)
+        add = cuda.Reduce(lambda x, y: x + y)
+        ones = np.ones(n, dtype=np.int32)
+        for trial in range(5):
+            a = cuda.to_device(ones, stream=sa)
+            sa.synchronize()
+            add(a, res=res, stream=sa)                     # queued on A, reads `a`
+            del a                                          # released while that kernel is queued / running
+            gc.collect()
+            b = cuda.device_array(n, np.int32, stream=sb)  # same size class
+            b.gpu_data.memset(0xFF, stream=sb)             # would corrupt the sum if it were the same block early
+            sb.synchronize()
+            sa.synchronize()
+            assert res.copy_to_host()[0] == n, trial
+            del b
+            gc.collect()
+            # both streams are idle now: the next request of this class comes from the pool
+            hits = mgr.stats()["hits"]
+            c = cuda.device_array(n, np.int32)
+            assert mgr.stats()["hits"] == hits + 1
+            del c
+            gc.collect()
+        assert mgr.stats()["hits"] >= 4
+    finally:
+        gc.collect()
+        ctx.reset()
+        ctx.memory_manager = original
+        cuda.current_context()
+
+
 def pool_via_the_environment_hook(cuda):
     from numba_cuda_amd import pool
     assert pool._numba_memory_manager is PoolMemoryManager
     assert PoolMemoryManager(context=None).interface_version == 1
 
 
-ALL = [pooled_arrays_reuse_blocks, pool_via_the_environment_hook]
+ALL = [pooled_arrays_reuse_blocks, a_block_in_use_on_another_stream_is_not_handed_out, pool_via_the_environment_hook]
