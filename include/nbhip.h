@@ -181,6 +181,11 @@ int nbh_transpose(const void *in, void *out, int64_t rows, int64_t cols, int64_t
  * destination must not overlap. */
 int nbh_assign(void *dst, const void *src, int ndim, const int64_t *shape, const int64_t *dst_strides,
                const int64_t *src_strides, int64_t itemsize, nbh_stream_t stream);
+/* The same assignment with ONE item as the right-hand side, passed by value (`value`
+ * points to `itemsize` bytes in HOST memory, read before the call returns; itemsize 1,
+ * 2, 4, 8 or 16): `darr[key] = scalar` without a device-side source. */
+int nbh_fill(void *dst, int ndim, const int64_t *shape, const int64_t *dst_strides, int64_t itemsize,
+             const void *value, nbh_stream_t stream);
 
 /* ---- xoroshiro128+ -------------------------------------------------------- */
 

@@ -64,6 +64,7 @@ SIGNATURES = {
     "nbh_reduce": (c_int, [c_int, c_int, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_size, c_vp]),
     "nbh_transpose": (c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "nbh_assign": (c_int, [c_vp, c_vp, c_int, P(c_i64), P(c_i64), P(c_i64), c_i64, c_vp]),
+    "nbh_fill": (c_int, [c_vp, c_int, P(c_i64), P(c_i64), c_i64, c_vp, c_vp]),
     "nbh_xoro_init_states": (c_int, [c_vp, c_i64, c_u64, c_u64, c_vp]),
     "nbh_xoro_uniform_f32": (c_int, [c_vp, c_i64, c_vp, c_i64, c_vp]),
     "nbh_xoro_uniform_f64": (c_int, [c_vp, c_i64, c_vp, c_i64, c_vp]),

@@ -116,6 +116,9 @@ def _normalise_shape(shape):
 
 # ---- the array types -------------------------------------------------------------------
 
+_FILL_ITEMSIZES = (1, 2, 4, 8, 16)   # what nbh_fill takes by value
+
+
 @functools.lru_cache(maxsize=1024)
 def _layout_of(shape, strides, itemsize):
     """The stride calculus object for an array that starts at offset 0.  Layout objects
@@ -447,6 +450,18 @@ class DeviceNDArray(DeviceNDArrayBase):
         if not _driver.is_device_memory(value) and not hasattr(value, "__cuda_array_interface__"):
             # host values take the dtype of the target, as a NumPy assignment would
             value = np.asarray(value).astype(self.dtype, copy=False)
+            if value.size == 1 and value.ndim <= lhs.ndim and self.dtype.itemsize in _FILL_ITEMSIZES:
+                # one item: it travels as a kernel argument, no device-side source needed
+                if lhs.ndim > _MAX_ASSIGN_NDIM:
+                    raise NotImplementedError("assignment supports at most %d axes" % _MAX_ASSIGN_NDIM)
+                item = np.ascontiguousarray(value).reshape(1)
+                vec = ctypes.c_int64 * max(lhs.ndim, 1)
+                _driver.driver.nbh_fill(lhs.device_ctypes_pointer.value, lhs.ndim, vec(*lhs.shape),
+                                        vec(*lhs.strides), self.dtype.itemsize, item.ctypes.data,
+                                        _driver._stream_handle(stream) or None)
+                if wait:
+                    stream.synchronize()
+                return
         rhs, _ = auto_device(value, stream=stream, user_explicit=True)
         if rhs.ndim > lhs.ndim:
             raise ValueError("Can't assign %s-D array to %s-D self" % (rhs.ndim, lhs.ndim))

@@ -239,6 +239,16 @@ class FakeLib:
         fn(user)                       # nothing is ever pending on the fake
         return 0
 
+    def nbh_fill(self, dst, ndim, shape, dst_strides, itemsize, value, stream):
+        """dst[...] = one item, as a broadcast assignment from the host copy of the item."""
+        keep = ctypes.create_string_buffer(ctypes.string_at(_addr(value), int(itemsize)), int(itemsize))
+        zeros = (ctypes.c_int64 * max(ndim, 1))(*([0] * max(ndim, 1)))
+        self._log("fill", _addr(dst), ndim, _addr(stream))
+        rc = self.nbh_assign(dst, ctypes.addressof(keep), ndim, shape, dst_strides, zeros, itemsize, stream)
+        self.calls.pop()          # the inner "assign" entry
+        self.calls.append(("assign", _addr(dst), 0, ndim, _addr(stream)))
+        return rc
+
     def nbh_assign(self, dst, src, ndim, shape, dst_strides, src_strides, itemsize, stream):
         """Strided broadcast assignment done with NumPy over raw host memory."""
         import numpy as np

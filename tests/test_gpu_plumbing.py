@@ -89,6 +89,36 @@ def test_flat_assignment_at_every_alignment(dtype):
             assert got.tobytes() == want.tobytes(), (n, d_off, s_off)
 
 
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float32, np.float64, np.complex128, np.bool_])
+def test_scalar_assignment_at_every_alignment_and_layout(dtype):
+    """`d[key] = scalar` passes the item by value: flat ranges from any offset (the
+    16-byte pattern must be in phase with the item), strided columns, blocks, 0-d."""
+    dt = np.dtype(dtype)
+    value = {"b": True, "c": 2.5 - 1.5j}.get(dt.kind, 77)
+    rng = np.random.default_rng(15)
+    base = rng.integers(0, 2, 5000 * dt.itemsize, dtype=np.uint8).view(dt) if dt.kind != "b" else np.zeros(5000, dt)
+    for lo, n in ((0, 5000), (1, 4999), (3, 17), (5, 1), (129, 3000), (7, 4093), (31, 33)):
+        want = base.copy()
+        d = cuda.to_device(want)
+        d[lo:lo + n] = value
+        want[lo:lo + n] = value
+        assert d.copy_to_host().tobytes() == want.tobytes(), (lo, n)
+    m = base[:4800].reshape(60, 80).copy()
+    d = cuda.to_device(m)
+    for key in ((slice(None), 3), (7, slice(None)), (slice(2, 50, 3), slice(1, 70, 7)), (slice(5, 55), slice(10, 20)),
+                (4, 9), slice(None)):
+        d[key] = value
+        m[key] = value
+        assert d.copy_to_host().tobytes() == m.tobytes(), key
+    z = cuda.to_device(np.zeros((), dt))
+    z[()] = value
+    assert z.copy_to_host()[()] == dt.type(value)
+    st = cuda.stream()
+    d.setitem(slice(None), 0, stream=st)
+    st.synchronize()
+    assert not d.copy_to_host().any()
+
+
 def test_large_pageable_copies_go_through_the_staging_ring():
     """Host copies of 32 MiB and more without a stream are pipelined through page-locked
     buffers by several threads: ragged sizes, odd offsets, fresh destination pages,
