@@ -347,8 +347,14 @@ class DeviceRecord(DeviceNDArrayBase):
             stream = devices.get_context().get_default_stream()
         field_type, offset = self.dtype.fields[key]
         target = type(self)(dtype=field_type, stream=stream, gpu_data=self.gpu_data.view(offset))
-        source, _ = auto_device(target.dtype.type(value), stream=stream)
-        _driver.device_to_device(target, source, source.dtype.itemsize, stream)
+        if target.dtype.itemsize in _FILL_ITEMSIZES and not target.dtype.fields and not target.dtype.shape:
+            item = np.asarray(value).astype(target.dtype).reshape(1)
+            none = (ctypes.c_int64 * 1)(0)
+            _driver.driver.nbh_fill(target.device_ctypes_pointer.value, 0, none, none, target.dtype.itemsize,
+                                    item.ctypes.data, _driver._stream_handle(stream) or None)
+        else:
+            source, _ = auto_device(target.dtype.type(value), stream=stream)
+            _driver.device_to_device(target, source, source.dtype.itemsize, stream)
         if wait:
             stream.synchronize()
 
