@@ -430,7 +430,13 @@ typedef nbh_u32x4 u32x4;
 // instruction covers eight whole 128-byte lines.  Within a wavefront LDS accesses
 // execute in program order; the wavefront-scope fences only keep the compiler
 // from moving them across the hand-over.
-template <typename Gen>
+// NT: non-temporal stores, chosen by the host when every run starts on a 128-byte line
+// (they are slower than cached stores when the packets of a wavefront straddle lines:
+// 31 float64 per generator 3.6 ms against 2.0 ms).  Runs that are not multiples of a
+// line reach 2.2-2.7 TB/s; cutting the rounds at the lines of the output instead (every
+// generator with its own offset) was tried and lost more in the generation loop than it
+// won in the stores.
+template <typename Gen, bool NT>
 __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__ states, int64_t n,
                                                           typename Gen::value_type *__restrict__ out,
                                                           int64_t count, const bm::LogTable *__restrict__ log_table)
@@ -503,15 +509,31 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
                 const int l = k * 8 + row;
                 if (l < lanes_here) {
                     u32x4 v = *reinterpret_cast<const u32x4 *>(&park[l][sub * PER]);
-                    nbh_store16<(int)sizeof(VT), true>(base + (int64_t)l * count + i0 + sub * PER, v);
+                    nbh_store16<(int)sizeof(VT), NT>(base + (int64_t)l * count + i0 + sub * PER, v);
                 }
             }
+        } else if (m % PER == 0) {
+            // a short round of whole packets: the lanes form rows x packets with the row
+            // length rounded up to a power of two, so no lane needs a division
+            const int packets = m / PER;
+            int shift = 0;
+            while ((1 << shift) < packets)
+                ++shift;
+            const int q = lane & ((1 << shift) - 1);
+            if (q < packets)
+                for (int l = lane >> shift; l < lanes_here; l += 64 >> shift) {
+                    u32x4 v = *reinterpret_cast<const u32x4 *>(&park[l][q * PER]);
+                    nbh_store16<(int)sizeof(VT), false>(base + (int64_t)l * count + i0 + q * PER, v);
+                }
         } else {
-            for (int f = lane; f < 64 * m; f += 64) {
-                const int l = f / m, j = f % m;
-                if (l < lanes_here)
+            // a ragged round: the same arrangement value by value
+            int shift = 0;
+            while ((1 << shift) < m)
+                ++shift;
+            const int j = lane & ((1 << shift) - 1);
+            if (j < m)
+                for (int l = lane >> shift; l < lanes_here; l += 64 >> shift)
                     base[(int64_t)l * count + i0 + j] = park[l][j];
-            }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -543,8 +565,14 @@ int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t 
             return rc;
     }
     nbh_pool_note_stream(nbh_hip_stream(stream));
-    hipLaunchKernelGGL((fill_kernel<Gen>), dim3((unsigned)grid), dim3(kFillBlock), 0, nbh_hip_stream(stream),
-                       (uint64_t *)states, n, (typename Gen::value_type *)out, count, log_table);
+    using VT = typename Gen::value_type;
+    const bool on_lines = ((uintptr_t)out % 128 == 0) && ((uint64_t)count * sizeof(VT)) % 128 == 0;
+    if (on_lines)
+        hipLaunchKernelGGL((fill_kernel<Gen, true>), dim3((unsigned)grid), dim3(kFillBlock), 0,
+                           nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);
+    else
+        hipLaunchKernelGGL((fill_kernel<Gen, false>), dim3((unsigned)grid), dim3(kFillBlock), 0,
+                           nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);
     return nbh_launch_status();
 }
 
