@@ -432,10 +432,9 @@ typedef nbh_u32x4 u32x4;
 // from moving them across the hand-over.
 // NT: non-temporal stores, chosen by the host when every run starts on a 128-byte line
 // (they are slower than cached stores when the packets of a wavefront straddle lines:
-// 31 float64 per generator 3.6 ms against 2.0 ms).  Runs that are not multiples of a
-// line reach 2.2-2.7 TB/s; cutting the rounds at the lines of the output instead (every
-// generator with its own offset) was tried and lost more in the generation loop than it
-// won in the stores.
+// 31 float64 per generator 3.6 ms against 2.0 ms).  Runs off the lines that are longer
+// than a line and a half go to fill_ring_kernel below (2^24 generators x 100 float64:
+// 5.1 ms here, 2.55 ms there); shorter ones and the compute-bound normal draws stay here.
 template <typename Gen, bool NT>
 __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__ states, int64_t n,
                                                           typename Gen::value_type *__restrict__ out,
@@ -545,6 +544,182 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
     }
 }
 
+// Runs that do not start on 128-byte lines (count * itemsize not a multiple of 128, or
+// an unaligned array) and are longer than a line.  Cutting the rounds where the runs
+// start makes every store of the kernel above straddle two lines.  Here the rounds of
+// the STORES follow the lines of the output instead, while generation still proceeds
+// 128 bytes per generator at a time: each lane parks its values in a ring of two
+// rounds, value i in column (i + skew) mod ring, where skew is the distance of the
+// run's start from the line below it.  After generation round r the columns of line r
+// are complete for every generator (the last `skew` values of the round wait in the
+// other half for line r+1), they start on a packet boundary of the ring whatever the
+// skew, and the wavefront stores them as whole, aligned, non-temporal 16-byte packets,
+// eight generators' lines per instruction.
+// The line in which one run ends is the line in which the next begins.  Each lane keeps
+// its first round in registers and, before the last lines are stored, adds the head of
+// its run to the ring of the generator before it, so that line too leaves as one whole
+// line; only the first line of a wavefront's first run and the last line of its last
+// run are stored value by value.  One more store-only round flushes the tails.
+// Requires count >= one round (the first round is drawn in the unrolled path).
+template <typename Gen>
+__global__ __launch_bounds__(kFillBlock) void fill_ring_kernel(uint64_t *__restrict__ states, int64_t n,
+                                                               typename Gen::value_type *__restrict__ out,
+                                                               int64_t count)
+{
+    static_assert(!Gen::kHeavy, "compute-bound generators gain nothing here and lose occupancy");
+    using VT = typename Gen::value_type;
+    constexpr int ROUND = 128 / (int)sizeof(VT);
+    constexpr int PER = 16 / (int)sizeof(VT);
+    constexpr int RING = 2 * ROUND;
+    constexpr int PITCH = RING + PER;  // 272-byte rows
+    __shared__ __attribute__((aligned(16))) VT ring_all[kFillBlock / 64][64][PITCH];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    VT(*ring)[PITCH] = ring_all[wave];
+    const int64_t t0 = ((int64_t)blockIdx.x * (kFillBlock / 64) + wave) * 64;
+    if (t0 >= n)
+        return;
+    const int64_t t = t0 + lane;
+    const bool live = t < n;
+    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+    uint64_t s0 = 0, s1 = 0;
+    if (live) {
+        u64x2 v = *reinterpret_cast<const u64x2 *>(states + 2 * t);
+        s0 = v.x;
+        s1 = v.y;
+    }
+    const int lanes_here = (n - t0 > 64) ? 64 : (int)(n - t0);
+    VT *__restrict__ base = out + t0 * count;
+    const int sub = lane & 7;
+    const int row = lane >> 3;
+    // position of generator l's run in values, modulo a line: (first + l * count) mod ROUND
+    const uint32_t first = (uint32_t)((uintptr_t)base / sizeof(VT));
+    const uint32_t step = (uint32_t)count;
+    const int my_skew = (int)((first + (uint32_t)lane * step) & (ROUND - 1));
+    const int64_t gen_rounds = (count + ROUND - 1) / ROUND;
+    VT head[ROUND];  // this lane's first round
+#pragma unroll
+    for (int j = 0; j < ROUND; ++j)
+        head[j] = VT(0);
+
+    for (int64_t r = 0; r <= gen_rounds; ++r) {
+        const int64_t i0 = r * ROUND;
+        const int half = (int)(r & 1) * ROUND;  // i0 mod RING
+        if (r < gen_rounds) {
+            const int m = (int)((count - i0 < ROUND) ? (count - i0) : ROUND);
+            const int col0 = half + my_skew;
+            if (m == ROUND) {
+                if (live) {
+                    VT val[ROUND];
+#pragma unroll
+                    for (int j = 0; j < ROUND; ++j)
+                        val[j] = Gen::draw(s0, s1, nullptr);
+#pragma unroll
+                    for (int j = 0; j < ROUND; ++j)
+                        ring[lane][(col0 + j) & (RING - 1)] = val[j];
+                    if (r == 0) {
+#pragma unroll
+                        for (int j = 0; j < ROUND; ++j)
+                            head[j] = val[j];
+                    }
+                }
+            } else if (live) {
+#pragma unroll 1
+                for (int j = 0; j < m; ++j)
+                    ring[lane][(col0 + j) & (RING - 1)] = Gen::draw(s0, s1, nullptr);
+            }
+            if (r == gen_rounds - 1 && live && lane > 0 && my_skew > 0) {
+                // the run before this one ends `my_skew` values into its last line: the
+                // rest of that line is the head of this run
+                const int skew_before = (int)((first + (uint32_t)(lane - 1) * step) & (ROUND - 1));
+                const int64_t last_line = (count + skew_before - my_skew) / ROUND;
+                const int at = (int)(last_line & 1) * ROUND + my_skew;
+#pragma unroll
+                for (int j = 0; j < ROUND; ++j)
+                    if (j < ROUND - my_skew)
+                        ring[lane - 1][at + j] = head[j];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // line r of every run: ring columns [half, half + ROUND), values from i0 - skew on
+        const int col = half + sub * PER;
+        if (r >= 1 && i0 + ROUND <= count) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int l = k * 8 + row;
+                if (l < lanes_here) {
+                    const int skew = (int)((first + (uint32_t)l * step) & (ROUND - 1));
+                    u32x4 v = *reinterpret_cast<const u32x4 *>(&ring[l][col]);
+                    nbh_store16<16, true>(base + (int64_t)l * count + (i0 - skew + sub * PER), v);
+                }
+            }
+        } else {
+            // first and last lines: whole packets first, all eight rows in flight at once
+            bool partial = false;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int l = k * 8 + row;
+                const int skew = (int)((first + (uint32_t)l * step) & (ROUND - 1));
+                const int64_t line_lo = i0 - skew;  // value index of the line's first column
+                // not past the end of the run; a first line shared with the run before is
+                // stored from that run's ring; the head of the next run completes a last line
+                const bool mine = l < lanes_here && line_lo < count && !(line_lo < 0 && l > 0);
+                const int64_t limit = (l + 1 < lanes_here) ? line_lo + ROUND : count;
+                const int64_t lo = line_lo + sub * PER;
+                const bool whole = lo >= 0 && lo + PER <= limit;
+                u32x4 v = *reinterpret_cast<const u32x4 *>(&ring[l & 63][col]);
+                if (mine && whole)
+                    nbh_store16<16, true>(base + (int64_t)l * count + lo, v);
+                partial |= mine && !whole;
+            }
+            if (partial) {
+                // the first line of the wavefront's first run, the last line of its last
+#pragma unroll 1
+                for (int k = 0; k < 8; ++k) {
+                    const int l = k * 8 + row;
+                    const int skew = (int)((first + (uint32_t)l * step) & (ROUND - 1));
+                    const int64_t line_lo = i0 - skew;
+                    if (l >= lanes_here || line_lo >= count || (line_lo < 0 && l > 0))
+                        continue;
+                    const int64_t limit = (l + 1 < lanes_here) ? line_lo + ROUND : count;
+                    const int64_t lo = line_lo + sub * PER;
+                    if (lo >= 0 && lo + PER <= limit)
+                        continue;
+                    for (int e = 0; e < PER; ++e)
+                        if (lo + e >= 0 && lo + e < limit)
+                            base[(int64_t)l * count + lo + e] = ring[l][col + e];
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if (live) {
+        u64x2 v = {s0, s1};
+        *reinterpret_cast<u64x2 *>(states + 2 * t) = v;
+    }
+}
+
+// runs from this many bytes on go through the ring when they are not on lines
+constexpr int64_t kRingFromBytes = 192;
+
+template <typename Gen, bool HEAVY = Gen::kHeavy>
+struct RingLaunch {
+    static void go(dim3 grid, hipStream_t s, uint64_t *states, int64_t n, typename Gen::value_type *out,
+                   int64_t count)
+    {
+        hipLaunchKernelGGL((fill_ring_kernel<Gen>), grid, dim3(kFillBlock), 0, s, states, n, out, count);
+    }
+};
+template <typename Gen>
+struct RingLaunch<Gen, true> {
+    static void go(dim3, hipStream_t, uint64_t *, int64_t, typename Gen::value_type *, int64_t) {}
+};
+
 template <typename Gen>
 int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t stream)
 {
@@ -570,6 +745,8 @@ int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t 
     if (on_lines)
         hipLaunchKernelGGL((fill_kernel<Gen, true>), dim3((unsigned)grid), dim3(kFillBlock), 0,
                            nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);
+    else if (!Gen::kHeavy && count * (int64_t)sizeof(VT) >= kRingFromBytes)
+        RingLaunch<Gen>::go(dim3((unsigned)grid), nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count);
     else
         hipLaunchKernelGGL((fill_kernel<Gen, false>), dim3((unsigned)grid), dim3(kFillBlock), 0,
                            nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);

@@ -95,26 +95,33 @@ def test_fill_against_oracle(n, kind, count):
 @pytest.mark.parametrize("kind", ["uniform_f32", "uniform_f64", "normal_f32", "normal_f64"])
 def test_fill_for_every_kind_of_round(kind):
     """Runs of every shape: whole rounds (128 bytes per generator), short rounds of whole
-    16-byte packets, ragged rounds, with the output starting on and off a 128-byte line
-    and a generator count that leaves the last wavefront partly empty."""
+    16-byte packets, ragged rounds, runs longer than a line that start anywhere in it,
+    with the output starting on and off a 128-byte line and generator counts that leave
+    the last wavefront partly empty."""
     dtype = np.float32 if kind.endswith("f32") else np.float64
     dist = nrandom.UNIFORM if kind.startswith("uniform") else nrandom.NORMAL
-    n = 300
-    host_states = cref.init_states(n, 7, 1)
-    for count in (1, 2, 3, 4, 8, 12, 15, 16, 17, 31, 32, 36, 48, 63, 64, 65, 100):
-        for lead in (0, 1):
-            _say("fill rounds", kind, count, lead)
-            states = cuda.to_device(host_states)
-            buf = cuda.device_array(n * count + lead, dtype=dtype)
-            out = buf[lead:]
-            nrandom.xoroshiro128p_fill(states, out, count, dist)
-            want, want_states = cref.fill(host_states, count, kind)
-            got = out.copy_to_host()
-            np.testing.assert_array_equal(states.copy_to_host(), want_states)
-            if dist == nrandom.UNIFORM:
-                assert got.tobytes() == want.tobytes(), (count, lead)
-            else:
-                assert _ulps(got, want).max() <= 2.0, (count, lead)      # tolerance: 2 ulp
+    for n in (300, 65, 1):
+        host_states = cref.init_states(n, 7, 1)
+        for count in (1, 2, 3, 4, 8, 12, 15, 16, 17, 24, 25, 31, 32, 33, 36, 47, 48, 49, 50, 63, 64, 65, 97, 100, 127,
+                      129, 250):
+            if n != 300 and count not in (3, 25, 50, 64, 97, 250):
+                continue
+            for lead in (0, 1, 5):
+                _say("fill rounds", kind, n, count, lead)
+                states = cuda.to_device(host_states)
+                # values before and after the runs must stay as they are
+                buf = cuda.to_device(np.full(n * count + lead + 40, -7, dtype=dtype))
+                out = buf[lead:lead + n * count]
+                nrandom.xoroshiro128p_fill(states, out, count, dist)
+                want, want_states = cref.fill(host_states, count, kind)
+                whole = buf.copy_to_host()
+                got = whole[lead:lead + n * count]
+                assert (whole[:lead] == -7).all() and (whole[lead + n * count:] == -7).all(), (n, count, lead)
+                np.testing.assert_array_equal(states.copy_to_host(), want_states)
+                if dist == nrandom.UNIFORM:
+                    assert got.tobytes() == want.tobytes(), (n, count, lead)
+                else:
+                    assert _ulps(got, want).max() <= 2.0, (n, count, lead)      # tolerance: 2 ulp
 
 
 def test_reference_statistics():
