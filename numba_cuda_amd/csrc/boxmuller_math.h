@@ -31,10 +31,13 @@ namespace bm {
 // and the table holds q_j = RN(1 / c_j) and t_j = -log(q_j) as a double-double, so that
 //     log(m) = t_j + log1p(r),  r = m * q_j - 1  (|r| <= 2^-8)
 // holds exactly.  t_hi keeps 42 fractional bits: e * ln2_hi + t_hi is then exact.
+// (The table also carries the two coefficient sets of the cosine, see below: it is the
+// one block of constants the generators keep in LDS.)
 struct LogTable {
     double q[128];
     double t_hi[128];
     double t_lo[128];
+    double trig[2][6];  // [0]: C6..C1 (cosine kernel), [1]: S6..S1 (sine kernel)
 };
 constexpr uint32_t kSqrtHalfBits = 0x3f3504f3u;  // float32 bits of sqrt(1/2)
 
@@ -59,6 +62,14 @@ inline void build_log_table(LogTable &t)
         t.q[j] = q;
         t.t_hi[j] = hi_part;
         t.t_lo[j] = (double)(full - (long double)hi_part);
+    }
+    const double c[6] = {-0x1.8fae9be8838d4p-37, 0x1.1ee9ebdb4b1c4p-29, -0x1.27e4f809c52adp-22,
+                         0x1.a01a019cb159p-16,   -0x1.6c16c16c15177p-10, 0x1.555555555554cp-5};
+    const double sn[6] = {0x1.5d93a5acfd57cp-33,  -0x1.ae5e68a2b9cebp-26, 0x1.71de357b1fe7dp-19,
+                          -0x1.a01a019c161d5p-13, 0x1.111111110f8a6p-7,   -0x1.5555555555549p-3};
+    for (int k = 0; k < 6; ++k) {
+        t.trig[0][k] = c[k];
+        t.trig[1][k] = sn[k];
     }
 }
 
@@ -120,9 +131,10 @@ BM_FN double bm_log_f32(float u, const LogTable *__restrict__ tab)
 //     sin(y0 + y1) = y0 + [ y0 z  (S1 + z (S2 + ... z S6)) + y1 (1 - z/2) ]
 //     cos(y0 + y1) = w  + [ z^2   (C1 + z (C2 + ... z C6)) + ((1 - w) - z/2) - y0 y1 ],  w = 1 - z/2
 // have the same shape, base + fma(factor, Horner(z), tail).  Double-precision
-// instructions are what bounds the generators, so the quadrant picks coefficients,
-// factor, tail and base per lane (32-bit selects) and ONE Horner chain runs.
-BM_FN double bm_cos_2pi(double x)
+// instructions are what bounds the generators, so ONE Horner chain runs: the quadrant
+// picks factor, tail and base per lane (32-bit selects) and the row of the coefficient
+// table (loads from LDS on the device, which cost the vector ALU nothing).
+BM_FN double bm_cos_2pi(double x, const LogTable *__restrict__ tab)
 {
     const double inv_pio2 = 0x1.45f306dc9c883p-1;
     const double pio2_1 = 0x1.921fb544p+0;             // first 33 bits of pi/2
@@ -138,17 +150,19 @@ BM_FN double bm_cos_2pi(double x)
     const double y1 = (r - y0) - w2;
 
     const bool odd = (n & 1) != 0;                     // odd quadrant: -+sin, even: +-cos
+    const double *__restrict__ k = tab->trig[n & 1];   // S6..S1 : C6..C1
     const double z = y0 * y0;
     const double hz = 0.5 * z;
     const double wc = 1.0 - hz;
-    double q = odd ? 0x1.5d93a5acfd57cp-33 : -0x1.8fae9be8838d4p-37;       // S6 : C6
-    q = __builtin_fma(z, q, odd ? -0x1.ae5e68a2b9cebp-26 : 0x1.1ee9ebdb4b1c4p-29);   // S5 : C5
-    q = __builtin_fma(z, q, odd ? 0x1.71de357b1fe7dp-19 : -0x1.27e4f809c52adp-22);   // S4 : C4
-    q = __builtin_fma(z, q, odd ? -0x1.a01a019c161d5p-13 : 0x1.a01a019cb159p-16);    // S3 : C3
-    q = __builtin_fma(z, q, odd ? 0x1.111111110f8a6p-7 : -0x1.6c16c16c15177p-10);    // S2 : C2
-    q = __builtin_fma(z, q, odd ? -0x1.5555555555549p-3 : 0x1.555555555554cp-5);     // S1 : C1
+    double q = __builtin_fma(z, k[0], k[1]);
+    q = __builtin_fma(z, q, k[2]);
+    q = __builtin_fma(z, q, k[3]);
+    q = __builtin_fma(z, q, k[4]);
+    q = __builtin_fma(z, q, k[5]);
     const double factor = z * (odd ? y0 : z);
-    const double tail = odd ? y1 * wc : __builtin_fma(-y0, y1, (1.0 - wc) - hz);
+    const double tail_sin = y1 * wc;
+    const double tail_cos = __builtin_fma(-y0, y1, (1.0 - wc) - hz);
+    const double tail = odd ? tail_sin : tail_cos;
     const double base = odd ? y0 : wc;
     const double pick = base + __builtin_fma(factor, q, tail);
     // cos(n*pi/2 + y): n&3 = 0: cos y, 1: -sin y, 2: -cos y, 3: sin y

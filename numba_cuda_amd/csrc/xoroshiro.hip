@@ -395,7 +395,7 @@ struct NormalF32 {
         const float two_pi = 6.283185307179586f;
         const float lg = (float)bm::bm_log_f32(u1, tab);
         const float r = sqrtf(-2.0f * lg);
-        const float c = (float)bm::bm_cos_2pi((double)(two_pi * u2));
+        const float c = (float)bm::bm_cos_2pi((double)(two_pi * u2), tab);
         return r * c;
     }
 };
@@ -411,7 +411,7 @@ struct NormalF64 {
         const double two_pi = 6.283185307179586;
         const float lg = (float)bm::bm_log_f32(u1, tab);
         const double r = sqrt(-2.0 * (double)lg);
-        const double c = bm::bm_cos_2pi(two_pi * (double)u2);
+        const double c = bm::bm_cos_2pi(two_pi * (double)u2, tab);
         return r * c;
     }
 };

@@ -50,7 +50,7 @@ int main(int argc, char **argv)
         for (uint32_t k = 0; k <= (1u << 24); k += stride) {
             const float u = (float)k * 0x1p-24f;
             const double x = variant == 0 ? 6.283185307179586 * (double)u : (double)(6.283185307179586f * u);
-            const double got = bm::bm_cos_2pi(x);
+            const double got = bm::bm_cos_2pi(x, &tab);
             const long double want = cosl((long double)x);
             const double err = (double)fabsl((long double)got - want) / ulp_of(want);
             if (err > worst)
@@ -68,7 +68,7 @@ int main(int argc, char **argv)
                 const float u = bm::bm_bits_to_float(((uint32_t)(127 - e) << 23) | mant);
                 const double x = 6.283185307179586 * (double)u;
                 const long double want = cosl((long double)x);
-                const double err = (double)fabsl((long double)bm::bm_cos_2pi(x) - want) / ulp_of(want);
+                const double err = (double)fabsl((long double)bm::bm_cos_2pi(x, &tab) - want) / ulp_of(want);
                 if (err > worst)
                     worst = err;
             }
