@@ -106,6 +106,17 @@ int nbh_host_get_device_pointer(void **dptr, void *hptr);
 /* cudadrv/driver.py:2496-2506 device_extents (cuMemGetAddressRange) */
 int nbh_mem_address_range(void **base, size_t *size, void *dptr);
 
+/* cudadrv/driver.py:861-878 GetIpcHandleMixin.get_ipc_handle (cuIpcGetMemHandle),
+ * :1408-1440 _CudaIpcImpl.open / close (cuIpcOpenMemHandle / cuIpcCloseMemHandle).
+ * `handle` is NBH_IPC_HANDLE_BYTES opaque bytes, valid in other processes on the same
+ * machine; `dptr` must be the start of an allocation.  nbh_ipc_open takes the number
+ * of bytes the importer will use.  Allocations of 2 GiB or more are refused
+ * (hipErrorNotSupported). */
+#define NBH_IPC_HANDLE_BYTES 64
+int nbh_ipc_get_handle(void *handle, void *dptr);
+int nbh_ipc_open(void **dptr, const void *handle, size_t nbytes);
+int nbh_ipc_close(void *dptr);
+
 /* cudadrv/driver.py:2625-2670 host_to_device / device_to_host / device_to_device:
  * stream == NULL selects the synchronous copy, any other stream the asynchronous
  * one, exactly as the reference picks cuMemcpyXtoY vs cuMemcpyXtoYAsync */

@@ -18,7 +18,8 @@ from numba_cuda_amd.core.errors import (CudaDriverError, CudaSupportError,  # no
 from numba_cuda_amd import cudadrv  # noqa: F401
 from numba_cuda_amd.cudadrv import devicearray, devices, driver  # noqa: F401
 from numba_cuda_amd.cudadrv.driver import (BaseCUDAMemoryManager, CudaAPIError,  # noqa: F401
-                                           HostOnlyCUDAMemoryManager, ManagedMemory, MemoryPointer, MappedMemory,
+                                           GetIpcHandleMixin, HostOnlyCUDAMemoryManager, IpcHandle,
+                                           ManagedMemory, MemoryPointer, MappedMemory,
                                            PinnedMemory, MemoryInfo, set_memory_manager)
 from numba_cuda_amd.cudadrv.devicearray import DeviceNDArray, DeviceRecord  # noqa: F401
 from numba_cuda_amd.api import *  # noqa: F401,F403

@@ -10,6 +10,7 @@ import os
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libnbhip.so")
+IPC_HANDLE_BYTES = 64      # NBH_IPC_HANDLE_BYTES
 
 c_int = ctypes.c_int
 c_i64 = ctypes.c_int64
@@ -44,6 +45,9 @@ SIGNATURES = {
     "nbh_host_unregister": (c_int, [c_vp]),
     "nbh_host_get_device_pointer": (c_int, [P(c_vp), c_vp]),
     "nbh_mem_address_range": (c_int, [P(c_vp), P(c_size), c_vp]),
+    "nbh_ipc_get_handle": (c_int, [c_vp, c_vp]),
+    "nbh_ipc_open": (c_int, [P(c_vp), c_vp, c_size]),
+    "nbh_ipc_close": (c_int, [c_vp]),
     "nbh_memcpy_h2d": (c_int, [c_vp, c_vp, c_size, c_vp]),
     "nbh_memcpy_d2h": (c_int, [c_vp, c_vp, c_size, c_vp]),
     "nbh_memcpy_d2d": (c_int, [c_vp, c_vp, c_size, c_vp]),

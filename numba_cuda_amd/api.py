@@ -159,6 +159,19 @@ def is_cuda_array(obj):
 
 
 @contextlib.contextmanager
+def open_ipc_array(handle, shape, dtype, strides=None, offset=0):
+    """Open an IPC memory handle given as its raw bytes (bytes, or a sequence of
+    ints) and yield it as a device array of `shape`, `dtype` and `strides` (1-d
+    C-contiguous when omitted); the mapping is closed when the block is left
+    (reference api.py:263-287)."""
+    dtype = np.dtype(dtype)
+    size = int(np.prod(shape)) * dtype.itemsize
+    ipchandle = driver.IpcHandle(None, driver.IpcMemHandle(handle), size, offset=offset)
+    yield ipchandle.open_array(_ctx(), shape=shape, strides=strides, dtype=dtype)
+    ipchandle.close()
+
+
+@contextlib.contextmanager
 def pinned(*arylist):
     "Temporarily page-lock the host arrays in `arylist`."
     ctx = _ctx()

@@ -2,6 +2,7 @@
 // passages to the HIP runtime.  The Python layer owns every lifetime.
 #include "common.h"
 
+
 #include <string.h>
 
 #include <atomic>
@@ -150,6 +151,44 @@ int nbh_mem_address_range(void **base, size_t *size, void *dptr)
         *size = n;
     return 0;
 }
+
+// ---- sharing an allocation with another process ---------------------------------------
+// Handles are hipIpcMemHandle_t, 64 opaque bytes.  Opening an allocation of 2 GiB or more
+// has been seen not to return on MI355X hosts, so such allocations are refused on both
+// sides (the exporter knows the size of the allocation, the importer only the size the
+// caller asks for).
+static_assert(sizeof(hipIpcMemHandle_t) == NBH_IPC_HANDLE_BYTES, "handle size");
+static constexpr size_t kIpcLimit = (size_t)2 << 30;
+
+int nbh_ipc_get_handle(void *handle, void *dptr)
+{
+    if (!handle || !dptr)
+        return (int)hipErrorInvalidValue;
+    hipDeviceptr_t base = nullptr;
+    size_t n = 0;
+    NBH_TRY(hipMemGetAddressRange(&base, &n, (hipDeviceptr_t)dptr));
+    if ((void *)base != dptr)
+        return (int)hipErrorInvalidValue;  // handles name whole allocations
+    if (n >= kIpcLimit)
+        return (int)hipErrorNotSupported;
+    hipIpcMemHandle_t h;
+    NBH_TRY(hipIpcGetMemHandle(&h, dptr));
+    memcpy(handle, &h, sizeof h);
+    return 0;
+}
+
+int nbh_ipc_open(void **dptr, const void *handle, size_t nbytes)
+{
+    if (!dptr || !handle)
+        return (int)hipErrorInvalidValue;
+    if (nbytes >= kIpcLimit)
+        return (int)hipErrorNotSupported;
+    hipIpcMemHandle_t h;
+    memcpy(&h, handle, sizeof h);
+    return (int)hipIpcOpenMemHandle(dptr, h, hipIpcMemLazyEnablePeerAccess);
+}
+
+int nbh_ipc_close(void *dptr) { return (int)hipIpcCloseMemHandle(dptr); }
 
 static int copy(void *dst, const void *src, size_t nbytes, hipMemcpyKind kind, nbh_stream_t stream)
 {

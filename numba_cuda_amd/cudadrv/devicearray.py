@@ -189,8 +189,9 @@ class DeviceNDArrayBase:
         return self.gpu_data
 
     def get_ipc_handle(self):
-        """An IpcArrayHandle built from whatever the context's memory manager returns
-        for this allocation (the built-in manager has no IPC support)."""
+        """An IpcArrayHandle - the memory manager's IPC handle for this allocation plus
+        the array's layout - that another process can open as a device array
+        (reference :331-340)."""
         handle = devices.get_context().get_ipc_handle(self.gpu_data)
         return IpcArrayHandle(ipc_handle=handle, array_desc=dict(shape=self.shape, strides=self.strides,
                                                                  dtype=self.dtype))

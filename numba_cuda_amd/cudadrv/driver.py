@@ -202,6 +202,15 @@ class Device:
         return {"pci_domain_id": self.PCI_DOMAIN_ID, "pci_bus_id": self.PCI_BUS_ID,
                 "pci_device_id": self.PCI_DEVICE_ID}
 
+    @classmethod
+    def from_identity(cls, identity):
+        """The device with this PCI identity (reference :489-503)."""
+        for dev in driver.list_devices():
+            if dev.get_device_identity() == identity:
+                return dev
+        raise RuntimeError("No device of {} is found. Target device may not be visible in this process."
+                           .format(identity))
+
     def get_primary_context(self):
         with self._ctx_lock:
             if self.primary_context is None:
@@ -417,7 +426,24 @@ class HostOnlyCUDAMemoryManager(BaseCUDAMemoryManager):
             yield
 
 
-class NumbaCUDAMemoryManager(HostOnlyCUDAMemoryManager):
+class GetIpcHandleMixin:
+    """A default get_ipc_handle() for managers whose memory comes from hipMalloc
+    (reference :861-878): the handle names the whole allocation, `offset` says where
+    in it `memory` starts."""
+
+    def get_ipc_handle(self, memory):
+        base, end = device_extents(memory)
+        if end - base >= IPC_ALLOCATION_LIMIT:
+            raise ValueError("allocations of 2 GiB or more cannot be shared between processes "
+                             "(this one has %d bytes)" % (end - base))
+        raw = ctypes.create_string_buffer(_lib.IPC_HANDLE_BYTES)
+        driver.nbh_ipc_get_handle(raw, base)
+        offset = int(memory.handle) - base
+        source_info = self.context.device.get_device_identity()
+        return IpcHandle(memory, IpcMemHandle(raw.raw), memory.size, source_info, offset=offset)
+
+
+class NumbaCUDAMemoryManager(GetIpcHandleMixin, HostOnlyCUDAMemoryManager):
     """Default manager: hipMalloc per allocation, deferred hipFree (reference
     :892-921)."""
 
@@ -441,9 +467,6 @@ class NumbaCUDAMemoryManager(HostOnlyCUDAMemoryManager):
         free, total = c_size_t(), c_size_t()
         driver.nbh_mem_info(byref(free), byref(total))
         return MemoryInfo(free=free.value, total=total.value)
-
-    def get_ipc_handle(self, memory):
-        raise NotImplementedError("IPC handles are not part of this build")
 
     @property
     def interface_version(self):
@@ -515,7 +538,21 @@ class Context:
         self.prepared = True
 
     def get_ipc_handle(self, memory):
+        """An IpcHandle for `memory`, to be sent to another process (reference :1190-1198)."""
+        if not sys.platform.startswith("linux"):
+            raise OSError("OS does not support CUDA IPC")
         return self.memory_manager.get_ipc_handle(memory)
+
+    def open_ipc_handle(self, handle, size):
+        """Map the allocation `handle` names into this process; `size` bytes of it
+        will be used (reference :1200-1209).  IpcHandle.close() unmaps it."""
+        dptr = c_void_p()
+        driver.nbh_ipc_open(byref(dptr), bytes(handle.reserved), size)
+        return MemoryPointer(context=weakref.proxy(self), pointer=dptr, size=size)
+
+    def can_access_peer(self, peer_device):
+        """One device per process here: only the device itself is reachable."""
+        return int(peer_device) == self.device.id
 
     def get_memory_info(self):
         return self.memory_manager.get_memory_info()
@@ -670,6 +707,132 @@ def _stream_finalizer(deallocs, handle):
 # --------------------------------------------------------------------------------
 # Memory objects
 # --------------------------------------------------------------------------------
+
+IPC_ALLOCATION_LIMIT = 2 << 30   # opening larger allocations has been seen to hang
+
+
+class IpcMemHandle:
+    """The 64 opaque bytes of a hipIpcMemHandle_t; `reserved` is what travels."""
+
+    def __init__(self, reserved=bytes(_lib.IPC_HANDLE_BYTES)):
+        self.reserved = reserved
+
+    @property
+    def reserved(self):
+        return self._reserved
+
+    @reserved.setter
+    def reserved(self, value):
+        value = bytes(bytearray(value))          # bytes, or any sequence of small ints
+        if len(value) != _lib.IPC_HANDLE_BYTES:
+            raise ValueError("an IPC memory handle has %d bytes, got %d" % (_lib.IPC_HANDLE_BYTES, len(value)))
+        self._reserved = value
+
+
+class _DirectIpc:
+    """An imported mapping of the exporter's allocation."""
+
+    def __init__(self, parent):
+        self.parent = parent
+        self._opened = None
+
+    def open(self, context):
+        p = self.parent
+        if p.base is not None:
+            raise ValueError("opening IpcHandle from original process")
+        if self._opened is not None:
+            raise ValueError("IpcHandle is already opened")
+        if p.offset + p.size >= IPC_ALLOCATION_LIMIT:
+            raise ValueError("allocations of 2 GiB or more cannot be shared between processes")
+        mem = context.open_ipc_handle(p.handle, p.offset + p.size)
+        self._opened = mem            # this object owns the mapping until close()
+        return mem.own().view(p.offset)
+
+    def close(self):
+        if self._opened is None:
+            raise ValueError("IpcHandle not opened")
+        driver.nbh_ipc_close(self._opened.handle)
+        self._opened = None
+
+
+class IpcHandle:
+    """A picklable name for a device allocation that another process on the same
+    machine can open (reference :1487-1603).
+
+    base        the exporter's memory, kept alive by the handle (None once pickled)
+    handle      IpcMemHandle
+    size        bytes of the shared region
+    source_info identity of the exporting device
+    offset      where the region starts in the underlying allocation
+    """
+
+    def __init__(self, base, handle, size, source_info=None, offset=0):
+        self.base = base
+        self.handle = handle
+        self.size = size
+        self.source_info = source_info
+        self.offset = offset
+        self._impl = None
+
+    def _sentry_source_info(self):
+        if self.source_info is None:
+            raise RuntimeError("IPC handle doesn't have source info")
+
+    def can_access_peer(self, context):
+        self._sentry_source_info()
+        if self.source_info == context.device.get_device_identity():
+            return True
+        return context.can_access_peer(Device.from_identity(self.source_info).id)
+
+    def open_staged(self, context):
+        """Copy through the exporting device when the importer cannot reach it.  That
+        needs a second device in the importing process, which this build never has."""
+        self._sentry_source_info()
+        if self._impl is not None:
+            raise ValueError("IpcHandle is already opened")
+        raise NotImplementedError("staged IPC between two devices is not part of this build")
+
+    def open_direct(self, context):
+        if self._impl is not None:
+            raise ValueError("IpcHandle is already opened")
+        self._impl = _DirectIpc(self)
+        try:
+            return self._impl.open(context)
+        except Exception:
+            self._impl = None
+            raise
+
+    def open(self, context):
+        """Map the memory into `context`'s process -> device memory pointer."""
+        if self.source_info is None or self.can_access_peer(context):
+            return self.open_direct(context)
+        return self.open_staged(context)
+
+    def open_array(self, context, shape, dtype, strides=None):
+        """open(), wrapped as a device array (1-d C-contiguous unless `strides` says otherwise)."""
+        from numba_cuda_amd.cudadrv import devicearray
+        if strides is None:
+            strides = dtype.itemsize
+        dptr = self.open(context)
+        return devicearray.DeviceNDArray(shape=shape, strides=strides, dtype=dtype, gpu_data=dptr)
+
+    def close(self):
+        if self._impl is None:
+            raise ValueError("IpcHandle not opened")
+        self._impl.close()
+        self._impl = None
+
+    def __reduce__(self):
+        return (_rebuild_ipc_handle, (self.__class__, self.handle.reserved, self.size, self.source_info, self.offset))
+
+    @classmethod
+    def _rebuild(cls, handle_bytes, size, source_info, offset):
+        return cls(base=None, handle=IpcMemHandle(handle_bytes), size=size, source_info=source_info, offset=offset)
+
+
+def _rebuild_ipc_handle(cls, *args):
+    return cls._rebuild(*args)
+
 
 class MemoryPointer:
     """A device buffer (reference :1606-1717).  `refct` counts the owned

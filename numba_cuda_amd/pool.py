@@ -26,7 +26,7 @@ from ctypes import byref, c_size_t, c_void_p
 from numba_cuda_amd.cudadrv import driver as _drv
 
 
-class PoolMemoryManager(_drv.HostOnlyCUDAMemoryManager):
+class PoolMemoryManager(_drv.GetIpcHandleMixin, _drv.HostOnlyCUDAMemoryManager):
     """Device allocations from the library's caching pool; host allocations as in the
     default manager."""
 
@@ -60,9 +60,6 @@ class PoolMemoryManager(_drv.HostOnlyCUDAMemoryManager):
         free, total = c_size_t(), c_size_t()
         _drv.driver.nbh_mem_info(byref(free), byref(total))
         return _drv.MemoryInfo(free=free.value, total=total.value)
-
-    def get_ipc_handle(self, memory):
-        raise NotImplementedError("IPC handles are not part of this build")
 
     def reset(self):
         super().reset()

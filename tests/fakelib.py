@@ -193,6 +193,34 @@ class FakeLib:
                 return 0
         return HIP_ERROR_INVALID_VALUE
 
+    # "other processes" are this process: a handle is the address, spelled in 64 bytes
+    def nbh_ipc_get_handle(self, handle, ptr):
+        addr = _addr(ptr)
+        if addr not in self.buffers:
+            return HIP_ERROR_INVALID_VALUE
+        raw = addr.to_bytes(8, "little") + b"fakelib!" + bytes(48)
+        ctypes.memmove(handle, raw, 64)
+        self._log("ipc_get_handle", addr)
+        return 0
+
+    def nbh_ipc_open(self, out, handle, nbytes):
+        raw = handle if isinstance(handle, bytes) else ctypes.string_at(_addr(handle), 64)
+        addr = int.from_bytes(raw[:8], "little")
+        if raw[8:16] != b"fakelib!" or addr not in self.buffers:
+            return HIP_ERROR_INVALID_VALUE
+        self.__dict__.setdefault("ipc_open", []).append(addr)
+        self._log("ipc_open", addr, int(nbytes))
+        self._out(out, addr)
+        return 0
+
+    def nbh_ipc_close(self, ptr):
+        addr = _addr(ptr)
+        if addr not in self.__dict__.get("ipc_open", []):
+            return HIP_ERROR_INVALID_VALUE
+        self.ipc_open.remove(addr)
+        self._log("ipc_close", addr)
+        return 0
+
     def _copy(self, kind, dst, src, nbytes, stream):
         self._log(kind, _addr(dst), _addr(src), int(nbytes), _addr(stream))
         ctypes.memmove(_addr(dst), _addr(src), int(nbytes))
