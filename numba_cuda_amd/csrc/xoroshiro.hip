@@ -598,6 +598,9 @@ __global__ __launch_bounds__(kFillBlock) void fill_ring_kernel(uint64_t *__restr
     const uint32_t step = (uint32_t)count;
     const int my_skew = (int)((first + (uint32_t)lane * step) & (ROUND - 1));
     const int64_t gen_rounds = (count + ROUND - 1) / ROUND;
+    // largest power of two (up to a packet) that divides the start of every run
+    const uint32_t both = (uint32_t)((uintptr_t)out / sizeof(VT)) | step;
+    const int grain = (both & 1) ? 1 : (both & 2) ? 2 : 4;
     VT head[ROUND];  // this lane's first round
 #pragma unroll
     for (int j = 0; j < ROUND; ++j)
@@ -611,22 +614,51 @@ __global__ __launch_bounds__(kFillBlock) void fill_ring_kernel(uint64_t *__restr
             const int col0 = half + my_skew;
             if (m == ROUND) {
                 if (live) {
-                    VT val[ROUND];
+                    union {
+                        VT val[ROUND];
+                        u32x4 pk[8];
+                        uint64_t pr[16];
+                    } mine;
 #pragma unroll
                     for (int j = 0; j < ROUND; ++j)
-                        val[j] = Gen::draw(s0, s1, nullptr);
+                        mine.val[j] = Gen::draw(s0, s1, nullptr);
+                    // every skew of the launch is a multiple of `grain` values: park in
+                    // pieces of that size (they neither straddle the wrap nor lose alignment)
+                    if (grain >= PER) {
 #pragma unroll
-                    for (int j = 0; j < ROUND; ++j)
-                        ring[lane][(col0 + j) & (RING - 1)] = val[j];
+                        for (int k = 0; k < 8; ++k)
+                            *reinterpret_cast<u32x4 *>(&ring[lane][(col0 + k * PER) & (RING - 1)]) = mine.pk[k];
+                    } else if (sizeof(VT) == 4 && grain >= 2) {
+#pragma unroll
+                        for (int k = 0; k < 16; ++k)
+                            *reinterpret_cast<uint64_t *>(&ring[lane][(col0 + 2 * k) & (RING - 1)]) = mine.pr[k];
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < ROUND; ++j)
+                            ring[lane][(col0 + j) & (RING - 1)] = mine.val[j];
+                    }
                     if (r == 0) {
 #pragma unroll
                         for (int j = 0; j < ROUND; ++j)
-                            head[j] = val[j];
+                            head[j] = mine.val[j];
                     }
                 }
             } else if (live) {
+                // the last, short round: four draws at a time so that the conversion of
+                // one overlaps the state update of the next
+                int j = 0;
 #pragma unroll 1
-                for (int j = 0; j < m; ++j)
+                for (; j + 4 <= m; j += 4) {
+                    VT four[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        four[e] = Gen::draw(s0, s1, nullptr);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        ring[lane][(col0 + j + e) & (RING - 1)] = four[e];
+                }
+#pragma unroll 1
+                for (; j < m; ++j)
                     ring[lane][(col0 + j) & (RING - 1)] = Gen::draw(s0, s1, nullptr);
             }
             if (r == gen_rounds - 1 && live && lane > 0 && my_skew > 0) {
