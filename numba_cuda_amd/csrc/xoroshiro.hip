@@ -204,7 +204,11 @@ __device__ __forceinline__ uint64_t next_d(uint64_t &s0, uint64_t &s1)
     const uint32_t sh_hi = funnel(t_hi, t_lo, 18), sh_lo = t_lo << 14;
     // rotl(t, 36): swap halves, then rotate left by 4
     const uint32_t r36_hi = funnel(t_lo, t_hi, 28), r36_lo = funnel(t_hi, t_lo, 28);
-    s0 = ((uint64_t)(r55_hi ^ t_hi ^ sh_hi) << 32) | (r55_lo ^ t_lo ^ sh_lo);
+    // a ^ b ^ c in one instruction (truth table 0x96); the compiler does not form it itself
+    // (the builtin returns int: without the casts the low word would be sign-extended)
+    const uint32_t n_hi = (uint32_t)__builtin_amdgcn_bitop3_b32(r55_hi, t_hi, sh_hi, 0x96);
+    const uint32_t n_lo = (uint32_t)__builtin_amdgcn_bitop3_b32(r55_lo, t_lo, sh_lo, 0x96);
+    s0 = ((uint64_t)n_hi << 32) | n_lo;
     s1 = ((uint64_t)r36_hi << 32) | r36_lo;
     return r;
 }
