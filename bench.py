@@ -37,8 +37,8 @@ MEASURED_TRAFFIC = {
     "copy_f32": 2147483648,
     # profiles/transpose_packets_f32_16384sq.txt: 1 073 769 401 B fetched + 1 074 524 157 B written
     "transpose_f32": 2148293558,
-    # profiles/xoroshiro_fill_and_init_2p24.txt: 268 536 188 B fetched + 4 564 907 203 B written
-    "rng_uniform_f32": 4833443391,
+    # profiles/xoroshiro_fill_and_init_2p24.txt: 268 618 773 B fetched + 4 563 547 721 B written
+    "rng_uniform_f32": 4832166494,
     # profiles/transpose_sheared_f64_12345x6789.txt: 1 026 969 245 B fetched + 670 744 593 B written
     "transpose_f64": 1697713838,
     # profiles/hbm_counters_other_workloads.txt

@@ -439,15 +439,18 @@ typedef nbh_u32x4 u32x4;
 // 31 float64 per generator 3.6 ms against 2.0 ms).  Runs off the lines that are longer
 // than a line and a half go to fill_ring_kernel below (2^24 generators x 100 float64:
 // 5.1 ms here, 2.55 ms there); shorter ones and the compute-bound normal draws stay here.
-template <typename Gen, bool NT>
+template <typename Gen, bool NT, int LINES>
 __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__ states, int64_t n,
                                                           typename Gen::value_type *__restrict__ out,
                                                           int64_t count, const bm::LogTable *__restrict__ log_table)
 {
     using VT = typename Gen::value_type;
-    constexpr int ROUND = 128 / (int)sizeof(VT);  // values per generator per round
+    constexpr int CHUNK = 128 / (int)sizeof(VT);  // values per line
+    constexpr int ROUND = LINES * CHUNK;          // values per generator per round
     constexpr int PER = 16 / (int)sizeof(VT);     // values per 16-byte packet
-    constexpr int PITCH = ROUND + PER;            // 144-byte rows
+    constexpr int PITCH = ROUND + PER;            // 144-byte rows (272 with two lines)
+    constexpr int LPR = 8 * LINES;                // lanes (packets) per row of a round
+    constexpr int RPI = 64 / LPR;                 // rows per store instruction
     __shared__ __attribute__((aligned(16))) VT park_all[kFillBlock / 64][64][PITCH];
 
     // the normal generators look their logarithm up in a 3 KiB table: into LDS first
@@ -478,23 +481,28 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
     }
     const int lanes_here = (n - t0 > 64) ? 64 : (int)(n - t0);  // generators this wavefront really has
     VT *__restrict__ base = out + t0 * count;
-    const int sub = lane & 7;   // which packet of a row this lane stores
-    const int row = lane >> 3;  // which of eight rows per store instruction
+    const int sub = lane % LPR;  // which packet of a row this lane stores
+    const int row = lane / LPR;  // which of the rows of a store instruction
 
     for (int64_t i0 = 0; i0 < count; i0 += ROUND) {
         const int m = (int)((count - i0 < ROUND) ? (count - i0) : ROUND);
-        if (m == ROUND && !Gen::kHeavy) {
+        if (m % CHUNK == 0 && !Gen::kHeavy) {
             if (live) {
-                union {
-                    VT val[ROUND];
-                    u32x4 pk[8];
-                } mine;
 #pragma unroll
-                for (int j = 0; j < ROUND; ++j)
-                    mine.val[j] = Gen::draw(s0, s1, nullptr);
+                for (int h = 0; h < LINES; ++h) {
+                    if (h * CHUNK >= m)  // the last round of a run may be short of lines
+                        break;
+                    union {
+                        VT val[CHUNK];
+                        u32x4 pk[8];
+                    } mine;
 #pragma unroll
-                for (int k = 0; k < 8; ++k)
-                    *reinterpret_cast<u32x4 *>(&park[lane][k * PER]) = mine.pk[k];
+                    for (int j = 0; j < CHUNK; ++j)
+                        mine.val[j] = Gen::draw(s0, s1, nullptr);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        *reinterpret_cast<u32x4 *>(&park[lane][h * CHUNK + k * PER]) = mine.pk[k];
+                }
             }
         } else if (live) {
             // transcendental-heavy draws stay in a rolled loop: unrolling sixteen
@@ -508,11 +516,24 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         if (m == ROUND) {
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int l = k * 8 + row;
+            for (int k = 0; k < LPR; ++k) {
+                const int l = k * RPI + row;
                 if (l < lanes_here) {
                     u32x4 v = *reinterpret_cast<const u32x4 *>(&park[l][sub * PER]);
                     nbh_store16<(int)sizeof(VT), NT>(base + (int64_t)l * count + i0 + sub * PER, v);
+                }
+            }
+        } else if (LINES > 1 && m % CHUNK == 0) {
+            // a last round of fewer whole lines: line by line, eight rows per instruction
+            for (int h = 0; h * CHUNK < m; ++h) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int l = k * 8 + (lane >> 3);
+                    if (l < lanes_here) {
+                        const int col = h * CHUNK + (lane & 7) * PER;
+                        u32x4 v = *reinterpret_cast<const u32x4 *>(&park[l][col]);
+                        nbh_store16<(int)sizeof(VT), NT>(base + (int64_t)l * count + i0 + col, v);
+                    }
                 }
             }
         } else if (m % PER == 0) {
@@ -778,13 +799,26 @@ int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t 
     nbh_pool_note_stream(nbh_hip_stream(stream));
     using VT = typename Gen::value_type;
     const bool on_lines = ((uintptr_t)out % 128 == 0) && ((uint64_t)count * sizeof(VT)) % 128 == 0;
-    if (on_lines)
-        hipLaunchKernelGGL((fill_kernel<Gen, true>), dim3((unsigned)grid), dim3(kFillBlock), 0,
+    // Lines per generator and round (measured, 2^24 generators, uniform draws): two lines
+    // beat one from 256-byte runs on (64 float32: 839 -> 754 us); four lines need 135 KB of
+    // LDS per workgroup, one workgroup per CU, which float32 generation only forgives when the
+    // runs are long (4 KiB on: 15.3 -> 12.9 ms at 1024 float32), float64 also at 512 B and 1 KiB.
+    const uint64_t run_bytes = (uint64_t)count * sizeof(VT);
+    const bool four = run_bytes >= 4096 || (sizeof(VT) == 8 && (run_bytes == 512 || run_bytes == 1024));
+    const int lines = Gen::kHeavy ? 1 : four ? 4 : run_bytes >= 256 ? 2 : 1;
+    if (on_lines && lines == 4)
+        hipLaunchKernelGGL((fill_kernel<Gen, true, 4>), dim3((unsigned)grid), dim3(kFillBlock), 0,
+                           nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);
+    else if (on_lines && lines == 2)
+        hipLaunchKernelGGL((fill_kernel<Gen, true, 2>), dim3((unsigned)grid), dim3(kFillBlock), 0,
+                           nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);
+    else if (on_lines)
+        hipLaunchKernelGGL((fill_kernel<Gen, true, 1>), dim3((unsigned)grid), dim3(kFillBlock), 0,
                            nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);
     else if (!Gen::kHeavy && count * (int64_t)sizeof(VT) >= kRingFromBytes)
         RingLaunch<Gen>::go(dim3((unsigned)grid), nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count);
     else
-        hipLaunchKernelGGL((fill_kernel<Gen, false>), dim3((unsigned)grid), dim3(kFillBlock), 0,
+        hipLaunchKernelGGL((fill_kernel<Gen, false, 1>), dim3((unsigned)grid), dim3(kFillBlock), 0,
                            nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);
     return nbh_launch_status();
 }

@@ -102,9 +102,13 @@ def test_fill_for_every_kind_of_round(kind):
     dist = nrandom.UNIFORM if kind.startswith("uniform") else nrandom.NORMAL
     for n in (300, 65, 1):
         host_states = cref.init_states(n, 7, 1)
+        # the last row: runs of whole lines, in rounds of one, two or four lines with every tail
         for count in (1, 2, 3, 4, 8, 12, 15, 16, 17, 24, 25, 31, 32, 33, 36, 47, 48, 49, 50, 63, 64, 65, 97, 100, 127,
-                      129, 250):
-            if n != 300 and count not in (3, 25, 50, 64, 97, 250):
+                      129, 250,
+                      80, 96, 128, 160, 512, 528, 544, 560, 1024, 1056, 1088, 1120):
+            if n != 300 and count not in (3, 25, 50, 64, 97, 250, 96, 560, 1120):
+                continue
+            if count > 250 and dist != nrandom.UNIFORM and count not in (512, 560):
                 continue
             for lead in (0, 1, 5):
                 _say("fill rounds", kind, n, count, lead)
