@@ -78,8 +78,8 @@ def is_contiguous(ary):
 def array_core(ary):
     """The part of a broadcast array that really exists in memory: index 0 along
     every zero-stride axis.  Contiguity and copies are decided on this core."""
-    if not ary.strides or not ary.size:
-        return ary
+    if not ary.strides or not ary.size or 0 not in ary.strides:
+        return ary          # nothing is repeated: the array is its own core
     picks = [slice(None) if stride else 0 for stride in ary.strides]
     return ary[tuple(picks)]
 
@@ -95,6 +95,8 @@ def check_array_compatibility(ary1, ary2):
     dtype, and same shape and strides once length-1 axes are dropped."""
     if ary1.dtype != ary2.dtype:
         raise TypeError("incompatible dtype: %s vs. %s" % (ary1.dtype, ary2.dtype))
+    if ary1.shape == ary2.shape and (ary1.strides == ary2.strides or not ary1.size):
+        return              # the common case needs no squeezed views
     sq1, sq2 = ary1.squeeze(), ary2.squeeze()
     if sq1.shape != sq2.shape:
         raise ValueError("incompatible shape: %s vs. %s" % (ary1.shape, ary2.shape))

@@ -516,6 +516,7 @@ class Context:
         self.memory_manager = _memory_manager(context=self)
         self.extras = {}
         self._scratch = {}   # stream handle -> device scratch for nbh_reduce
+        self._result_slots = {}   # stream handle -> host-mapped slot for results that go back to the caller
 
     @property
     def memory_manager(self):
@@ -530,6 +531,7 @@ class Context:
     def reset(self):
         _logger.info("reset context of device %s", self.device.id)
         self._scratch.clear()
+        self._free_result_slots()
         self.memory_manager.reset()
         self.deallocations.clear()
 
@@ -622,6 +624,33 @@ class Context:
             driver.nbh_memset8(ptr, 0, nbytes + self._RESULT_SLOT_BYTES, None)
             entry = self._scratch[stream_handle] = (ptr, ptr + nbytes, nbytes, mem)
         return entry[0], entry[1], entry[2]
+
+    def reduce_result_slot(self, stream_handle, dtype):
+        """(device-visible address, one-item host array) of a result slot in page-locked,
+        device-mapped host memory: a reduction that returns its value to the caller
+        writes it there, and the host reads it after waiting for the stream - no
+        device-to-host copy (which costs as much again as the launch).  One slot per
+        stream, viewed through the dtype asked for."""
+        entry = self._result_slots.get(stream_handle)
+        if entry is None:
+            host = c_void_p()
+            driver.nbh_host_alloc(byref(host), self._RESULT_SLOT_BYTES, 2)       # 2: device-mapped
+            dev = c_void_p()
+            driver.nbh_host_get_device_pointer(byref(dev), host.value)
+            raw = np.frombuffer((ctypes.c_ubyte * self._RESULT_SLOT_BYTES).from_address(host.value), dtype=np.uint8)
+            entry = self._result_slots[stream_handle] = (dev.value, host.value, raw, {})
+        view = entry[3].get(dtype)
+        if view is None:
+            view = entry[3][dtype] = entry[2][:dtype.itemsize].view(dtype)
+        return entry[0], view
+
+    def _free_result_slots(self):
+        slots, self._result_slots = self._result_slots, {}
+        for _, host, _, _ in slots.values():
+            try:
+                driver.nbh_host_free(host)
+            except Exception:
+                pass
 
     def __repr__(self):
         return "<HIP context of device %d>" % self.device.id

@@ -198,13 +198,14 @@ class Reduce:
             arr, _ = devicearray.auto_device(arr, stream=stream)
 
         hstream = stream.handle if type(stream) is _driver.Stream else _driver._stream_handle(stream)
-        scratch_ptr, slot, scratch_bytes = ctx.reduce_scratch(hstream)
+        scratch_ptr, _, scratch_bytes = ctx.reduce_scratch(hstream)
         if res is not None:
             if res.dtype != dtype:
                 raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
             out_ptr = res.device_ctypes_pointer.value
         else:
-            out_ptr = slot      # per-stream result slot: no allocation per call
+            # per-stream slot in host memory the device can write: no allocation, no copy back
+            out_ptr, host_view = ctx.reduce_result_slot(hstream, dtype)
         init_ptr = _init_buffer(dtype, init)
         drv = _driver.driver
         rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size,
@@ -214,12 +215,9 @@ class Reduce:
             drv.check("nbh_reduce", rc)
         if res is not None:
             return None
-        # the value is wanted on the host now: wait for the stream, then fetch it
-        if hstream:
-            drv.nbh_stream_synchronize(hstream)
-        host = np.empty(1, dtype=dtype)
-        drv.nbh_memcpy_d2h(host.ctypes.data, out_ptr, dtype.itemsize, None)
-        return host[0]
+        # the value is wanted on the host now: wait for the stream, then read the slot
+        drv.nbh_stream_synchronize(hstream or None)
+        return host_view[0]
 
 
 _DTYPE_CODE = {np.dtype(name): code for name, code in _lib.DTYPE_CODES.items()}
