@@ -113,5 +113,6 @@ def test_pooled_memory_can_be_shared(worker):
         np.testing.assert_array_equal(fut.result(timeout=TIMEOUT), arr[100:])
         del devarr
     finally:
+        ctx.memory_manager.reset()              # hands the idle blocks back to the driver
         ctx.memory_manager = original
         cuda.current_context()
