@@ -4,13 +4,14 @@
 // The host first squeezes the index space: axes of length 1 vanish and neighbouring
 // axes that are laid out back to back on both sides fuse.  What is left decides
 // the kernel:
-//   * one axis with unit stride on both sides -> a flat copy: one workgroup per
-//     16 KiB, 16-byte packets, four loads in flight per lane, non-temporal on both
-//     sides; packets start at the first 128-byte line of the destination, the bytes
+//   * one axis with unit stride on both sides -> a flat copy: one wavefront per
+//     workgroup and one 16-byte packet per lane (1 KiB per workgroup), non-temporal on
+//     both sides; packets start at the first 128-byte line of the destination, the bytes
 //     in front of it and behind the last packet are done chunk by chunk.  Measured on
 //     MI355X, 2^28 float32, TB/s: a fixed grid looping grid-stride with cached
 //     accesses 4.80, non-temporal 5.03, a fixed grid looping over contiguous slices
-//     5.5, one workgroup per 16 KiB 6.4 (hipMemcpyDtoD: 5.2)
+//     5.5, one workgroup of 256 lanes per 16 KiB 6.3, per 4 KiB 6.6, one wavefront per
+//     1 KiB 6.7 (hipMemcpyDtoD: 5.2)
 //   * two axes, the inner one with unit stride on both sides (a block of a pitched
 //     matrix, `d[10:1000, 20:4000] = s`) -> every row is a run of bytes moved in 16-byte
 //     packets that need only the alignment the rows have; a workgroup is TY rows x TX
@@ -45,42 +46,42 @@ template <> struct ChunkOf<16> { using type = Chunk16; };
 
 typedef nbh_u32x4 u32x4;
 
+// Streaming kernels do best here with the smallest workgroups: one wavefront, one 16-byte
+// packet per lane, 1 KiB per workgroup, in launch order (2^28 float32 copied, TB/s: 256 lanes x 4
+// packets 6.1-6.3, 256 x 2 6.0, 256 x 1 6.6, 64 x 1 6.7-6.8; filled: 256 x 16 4.9, x 4 5.9, x 1 6.6,
+// 64 x 1 4.8).
+constexpr int kFlatThreads = 64;
+
 template <int G>
-__global__ __launch_bounds__(kThreads) void copy_flat(char *__restrict__ dst, const char *__restrict__ src,
-                                                      int64_t nbytes, int64_t head)
+__global__ __launch_bounds__(kFlatThreads) void copy_flat(char *__restrict__ dst, const char *__restrict__ src,
+                                                          int64_t nbytes, int64_t head)
 {
-    constexpr int kInFlight = 4;
     const int64_t npack = (nbytes - head) / 16;
     const char *__restrict__ from = src + head;  // packets: G-aligned here,
     char *__restrict__ to = dst + head;           // 128-byte aligned here
-    const int64_t p0 = (int64_t)blockIdx.x * (kThreads * kInFlight) + threadIdx.x;
-    u32x4 v[kInFlight];
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u)
-        if (p0 + u * kThreads < npack)
-            v[u] = nbh_load16<G, true>(from + (p0 + u * kThreads) * 16);
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u)
-        if (p0 + u * kThreads < npack)
-            nbh_store16<16, true>(to + (p0 + u * kThreads) * 16, v[u]);
+    const int64_t p = (int64_t)blockIdx.x * kFlatThreads + threadIdx.x;
+    if (p < npack)
+        nbh_store16<16, true>(to + p * 16, nbh_load16<G, true>(from + p * 16));
 
     if (blockIdx.x == 0) {  // fewer than 128 + 16 bytes in all
         using C = typename ChunkOf<G>::type;
-        for (int64_t b = (int64_t)threadIdx.x * G; b < head; b += (int64_t)kThreads * G)
+        for (int64_t b = (int64_t)threadIdx.x * G; b < head; b += (int64_t)kFlatThreads * G)
             *reinterpret_cast<C *>(dst + b) = *reinterpret_cast<const C *>(src + b);
-        for (int64_t b = head + npack * 16 + (int64_t)threadIdx.x * G; b < nbytes; b += (int64_t)kThreads * G)
+        for (int64_t b = head + npack * 16 + (int64_t)threadIdx.x * G; b < nbytes; b += (int64_t)kFlatThreads * G)
             *reinterpret_cast<C *>(dst + b) = *reinterpret_cast<const C *>(src + b);
     }
 }
 
 // Rows of `run` bytes, `rows` of them, row r at dst + r * dst_pitch / src + r * src_pitch.
 // tx_log2: lanes along a row per workgroup = 1 << tx_log2; segs: workgroups along a row.
+constexpr int kRowsInFlight = 1;  // packets per lane (16384 x 16000 float32 block: 4 -> 6.2 TB/s, 2 -> 6.0, 1 -> 6.6)
+
 template <int G, bool NT>
 __global__ __launch_bounds__(kThreads) void copy_rows(char *__restrict__ dst, const char *__restrict__ src,
                                                       int64_t rows, int64_t run, int64_t dst_pitch,
                                                       int64_t src_pitch, int tx_log2, int64_t segs)
 {
-    constexpr int kInFlight = 4;
+    constexpr int kInFlight = kRowsInFlight;
     const int tx_count = 1 << tx_log2;
     const int tx = threadIdx.x & (tx_count - 1), ty = threadIdx.x >> tx_log2;
     const int64_t seg = (int64_t)blockIdx.x % segs;
@@ -141,18 +142,17 @@ __global__ __launch_bounds__(kThreads) void copy_strided(char *__restrict__ dst,
 // `pattern` is the item repeated to 16 bytes (item sizes 1, 2, 4, 8, 16), rotated so that
 // it is right at every 16-byte boundary of the destination.
 
+// (a pure write is limited by the rate at which workgroups start before one wavefront per
+// workgroup pays: four wavefronts, one packet per lane, 4 KiB per workgroup)
 template <int G>
 __global__ __launch_bounds__(kThreads) void fill_flat(char *__restrict__ dst, int64_t nbytes, int64_t head,
-                                                      u32x4 pattern, u32x4 unrotated)
+                                                          u32x4 pattern, u32x4 unrotated)
 {
-    constexpr int kInFlight = 4;
     const int64_t npack = (nbytes - head) / 16;
     char *__restrict__ to = dst + head;  // 128-byte aligned
-    const int64_t p0 = (int64_t)blockIdx.x * (kThreads * kInFlight) + threadIdx.x;
-#pragma unroll
-    for (int u = 0; u < kInFlight; ++u)
-        if (p0 + u * kThreads < npack)
-            nbh_store16<16, true>(to + (p0 + u * kThreads) * 16, pattern);
+    const int64_t p = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (p < npack)
+        nbh_store16<16, true>(to + p * 16, pattern);
     if (blockIdx.x == 0) {  // in front of the first line and behind the last packet
         using C = typename ChunkOf<G>::type;
         union {
@@ -201,12 +201,12 @@ template <int G> int launch_flat(void *dst, const void *src, int64_t nbytes, hip
     int64_t head = (int64_t)((128 - (uintptr_t)dst % 128) % 128);
     if (head > nbytes)
         head = nbytes;
-    int64_t grid = ((nbytes - head) / 16 + 4 * kThreads - 1) / (4 * kThreads);
+    int64_t grid = ((nbytes - head) / 16 + kFlatThreads - 1) / kFlatThreads;
     if (grid < 1)
         grid = 1;
     if (grid > 0x7fffffffLL)
         return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL((copy_flat<G>), dim3((unsigned)grid), dim3(kThreads), 0, s, (char *)dst, (const char *)src,
+    hipLaunchKernelGGL((copy_flat<G>), dim3((unsigned)grid), dim3(kFlatThreads), 0, s, (char *)dst, (const char *)src,
                        nbytes, head);
     return nbh_launch_status();
 }
@@ -219,7 +219,7 @@ int launch_rows(void *dst, const void *src, int64_t rows, int64_t run, int64_t d
     int tx_log2 = 0;
     while (tx_log2 < 8 && (1 << tx_log2) < npack)
         ++tx_log2;
-    const int64_t per_seg = (int64_t)(1 << tx_log2) * 4;
+    const int64_t per_seg = (int64_t)(1 << tx_log2) * kRowsInFlight;
     int64_t segs = (npack + per_seg - 1) / per_seg;
     if (segs < 1)
         segs = 1;
@@ -266,7 +266,7 @@ template <int G> int launch_fill_flat(void *dst, int64_t nbytes, int64_t itemsiz
         plain.b[k] = item[k % itemsize];
         rotated.b[k] = item[(head + k) % itemsize];
     }
-    int64_t grid = ((nbytes - head) / 16 + 4 * kThreads - 1) / (4 * kThreads);
+    int64_t grid = ((nbytes - head) / 16 + kThreads - 1) / kThreads;
     if (grid < 1)
         grid = 1;
     if (grid > 0x7fffffffLL)
