@@ -31,8 +31,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E published peak
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (see profiles/); filled in per workload once measured, else None
 MEASURED_TRAFFIC = {
-    # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 779 029 B fetched + 32 832 B written
-    "reduce_f32_sum": 1073811861,
+    # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 780 027 B fetched + 32 832 B written
+    "reduce_f32_sum": 1073812859,
     # profiles/copy_flat_f32_2p28.txt: the calibration kernel itself
     "copy_f32": 2147483648,
     # profiles/transpose_packets_f32_16384sq.txt: 1 073 769 401 B fetched + 1 074 524 157 B written

@@ -19,13 +19,19 @@
 // release RMW would emit) writes back the whole L2 of the XCD; measured on MI355X
 // that costs about 90 us per 2048 workgroups on a 160 us kernel.  It is also more
 // than is needed: the only datum to publish is the partial itself.  So the partial
-// is written with an agent-scope atomic store (written through to where every XCD
-// sees it), the wavefront then waits until that store has been acknowledged (a
-// workgroup-scope release fence is exactly that wait and nothing else), and only
-// then takes its ticket with a relaxed agent-scope atomic add.  The finishing
-// workgroup invalidates its caches once (agent-scope acquire fence) and reads the
-// partials with agent-scope atomic loads.  Few, large workgroups keep the tickets,
-// which all hit one address, off the critical path.
+// is put in place with an agent-scope atomic EXCHANGE - a read-modify-write is carried
+// out where every XCD looks, and its result comes back from there - the wavefront
+// waits for that result, and only then takes its ticket with a relaxed agent-scope
+// atomic add.  (A written-through atomic store followed by a wait for its
+// acknowledgement is not enough: the acknowledgement does not mean that the value is
+// where other XCDs read it.  With tickets and partials in different pages a ticket was
+// seen to overtake its partial, one wrong sum in some 10^4 closings; the exchange costs
+// 0.4 us on a 154 us kernel.)  The finishing workgroup invalidates its caches once
+// (agent-scope acquire fence) and reads the partials with agent-scope atomic loads.
+// Few, large workgroups keep the tickets, which all hit one address, off the critical
+// path: atomics on one address - or on neighbouring addresses, which share a memory
+// channel - take about 6 ns each, one after the other (one workgroup per 16 KiB with
+// tickets 4 bytes apart: 557 us for 2^28 float32; tickets 4 KiB apart: 180 us).
 //
 // HBM roofline: n * itemsize bytes are read once; nothing else of size is moved.
 #include "common.h"
@@ -282,12 +288,16 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
     Word *partials = reinterpret_cast<Word *>(partials_raw);
     if (tid == 0) {
         const Image img = __builtin_bit_cast(Image, total);
+        Word before[kWords];
 #pragma unroll
         for (int w = 0; w < kWords; ++w)
-            __hip_atomic_store(&partials[(int64_t)blockIdx.x * kWords + w], img.w[w], __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-        // wait for the write-through store to be acknowledged before the ticket is drawn
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            before[w] = __hip_atomic_exchange(&partials[(int64_t)blockIdx.x * kWords + w], img.w[w], __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+        // the results of the exchanges come from where every XCD looks: once they are
+        // back, the partial is in place and the ticket may be drawn
+#pragma unroll
+        for (int w = 0; w < kWords; ++w)
+            asm volatile("" ::"v"(before[w]) : "memory");
         unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last_block = (t == gridDim.x - 1);
         if (last_block)  // every partial has been published: drop stale cache lines once

@@ -88,7 +88,8 @@ def test_every_operator_and_dtype_against_oracle(op, sfx):
                "max": lambda a, b: max(a, b), "min": lambda a, b: min(a, b)}[op]
     red = cuda.Reduce(functor)
     rng = np.random.default_rng(abs(hash((op, sfx))) % 2**32)
-    for n in (1, 7, 64, 65, 255, 256, 257, 4096, 65536, 300001, 2**21 + 3):
+    # the last size is past 16 MiB for every element type: every workgroup loops over its slice
+    for n in (1, 7, 64, 65, 255, 256, 257, 4096, 65536, 300001, 2**21 + 3, 2**24 + 5):
         _say("reduce", op, sfx, n)
         if dt.kind == "f":
             a = rng.standard_normal(n).astype(dt) if op != "mul" else (1 + rng.standard_normal(n) * 1e-3).astype(dt)
@@ -174,6 +175,11 @@ def test_runs_are_bitwise_reproducible():
     first = sum_reduce(a)
     for _ in range(10):
         assert sum_reduce(a).tobytes() == first.tobytes()
+    # past 16 MiB, where the workgroups loop
+    b = cuda.to_device(rng.standard_normal(20_000_003).astype(np.float32))
+    first = sum_reduce(b)
+    for _ in range(20):
+        assert sum_reduce(b).tobytes() == first.tobytes()
 
 
 def test_stream_and_result_slot_round_robin():
@@ -233,18 +239,18 @@ def test_fullsize_int64_sum_2_pow_28_bit_exact():
     assert got == cref.tree("add", a) == a.sum()
 
 
-def test_back_to_back_reductions_never_see_stale_partials():
+@pytest.mark.parametrize("n_min,n_max,calls", [(5000, 3_000_000, 3000), (2_200_000, 9_000_000, 1500)])
+def test_back_to_back_reductions_never_see_stale_partials(n_min, n_max, calls):
     """Thousands of launches reuse one scratch buffer per stream with different
     data each time; a partial read from a stale cache line would change an integer
-    sum.  Sizes span 2 to 512 workgroups."""
+    sum.  Sizes span 2 to 512 workgroups; in the second case every launch has all 512
+    and they finish close together."""
     rng = np.random.default_rng(77)
-    n_max = 3_000_000
     base = rng.integers(-2**40, 2**40, n_max + 4096, dtype=np.int64)
     d = cuda.to_device(base)
-    calls = 3000
     offs = rng.integers(0, 4096, calls)
-    sizes = rng.integers(5000, n_max, calls)
-    sizes[::7] = rng.integers(2_500_000, n_max, len(sizes[::7]))
+    sizes = rng.integers(n_min, n_max, calls)
+    sizes[::7] = rng.integers(max(n_min, 2_500_000), n_max, len(sizes[::7]))
     out = cuda.device_array(calls, np.int64)
     streams = [cuda.stream() for _ in range(3)]
     for i in range(calls):
