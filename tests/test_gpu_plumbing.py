@@ -120,13 +120,16 @@ def test_scalar_assignment_at_every_alignment_and_layout(dtype):
 
 
 def test_large_pageable_copies_go_through_the_staging_ring():
-    """Host copies of 32 MiB and more without a stream are pipelined through page-locked
-    buffers by several threads: ragged sizes, odd offsets, fresh destination pages,
-    two Python threads at once, and the ordering hipMemcpy gives after work on a stream."""
+    """Host copies from a few MiB on are pipelined through page-locked buffers by several
+    threads, in chunks of a quarter of the copy (1 to 16 MiB): sizes around every threshold
+    and chunk size, ragged sizes, odd offsets, fresh destination pages, Python threads at
+    once, and the ordering hipMemcpy gives after work on a stream."""
     import threading
     rng = np.random.default_rng(14)
     big = rng.integers(0, 255, (80 << 20) + 12345, dtype=np.uint8)
-    for lo, n in ((0, big.size), (1, (32 << 20)), (4097, (48 << 20) + 1), (3, (32 << 20) - 1)):
+    for lo, n in ((0, big.size), (1, (32 << 20)), (4097, (48 << 20) + 1), (3, (32 << 20) - 1),
+                  (0, (2 << 20) - 1), (5, 2 << 20), (0, (2 << 20) + 1), (7, (4 << 20) + 3), (1, (8 << 20) - 1),
+                  (2, 8 << 20), (0, (9 << 20) + 17), (3, (16 << 20) + 1), (0, (64 << 20) + 1), (9, 1 << 20)):
         src = big[lo:lo + n]
         d = cuda.to_device(src)                                  # pageable -> device
         back = d.copy_to_host()                                  # device -> fresh pageable memory
