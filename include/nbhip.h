@@ -45,8 +45,10 @@ enum nbh_dtype {
  * JIT gives the Python functor (cpython/builtins.py:224-269):
  *   ADD a + b, MUL a * b      native arithmetic, integers wrap modulo 2^bits; complex
  *                             products are (ac - bd) + (ad + bc)i, each operation rounded
- *   MAX b if b > a else a,  MIN b if b < a else a */
-enum nbh_op { NBH_ADD = 0, NBH_MUL = 1, NBH_MAX = 2, NBH_MIN = 3, NBH_OP_COUNT = 4 };
+ *   MAX b if b > a else a,  MIN b if b < a else a
+ *   AND a & b, OR a | b, XOR a ^ b     integer element types only */
+enum nbh_op { NBH_ADD = 0, NBH_MUL = 1, NBH_MAX = 2, NBH_MIN = 3, NBH_AND = 4, NBH_OR = 5, NBH_XOR = 6,
+              NBH_OP_COUNT = 7 };
 
 /* ---- library / device ---------------------------------------------------- */
 

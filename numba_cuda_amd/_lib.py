@@ -80,7 +80,7 @@ SIGNATURES = {
 DTYPE_CODES = {"int8": 0, "int16": 1, "int32": 2, "int64": 3,
                "uint8": 4, "uint16": 5, "uint32": 6, "uint64": 7,
                "float32": 8, "float64": 9, "complex64": 10, "complex128": 11}
-OP_CODES = {"add": 0, "mul": 1, "max": 2, "min": 3}
+OP_CODES = {"add": 0, "mul": 1, "max": 2, "min": 3, "and": 4, "or": 5, "xor": 6}
 
 # hipError_t values the Python layer branches on
 HIP_SUCCESS = 0

@@ -82,13 +82,24 @@ struct OpMax {
 struct OpMin {
     template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return b < a ? b : a; }
 };
+// bitwise functors, integers only
+struct OpAnd {
+    template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a & b; }
+};
+struct OpOr {
+    template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a | b; }
+};
+struct OpXor {
+    template <typename A> static __device__ __forceinline__ A apply(A a, A b) { return a ^ b; }
+};
+template <typename Op> struct IsBitwise : std::integral_constant<bool, std::is_same<Op, OpAnd>::value || std::is_same<Op, OpOr>::value || std::is_same<Op, OpXor>::value> {};
 
 // Accumulator type.  Sums and products of integers are carried in an unsigned
 // type at least 32 bits wide: arithmetic modulo 2^32 / 2^64 truncates to the same
 // element value as arithmetic modulo 2^bits, and unsigned wrap-around is defined.
 // Comparisons keep the signedness of the element type.
 template <typename T, typename Op> struct AccOf {
-    static constexpr bool arith = std::is_same<Op, OpAdd>::value || std::is_same<Op, OpMul>::value;
+    static constexpr bool arith = std::is_same<Op, OpAdd>::value || std::is_same<Op, OpMul>::value || IsBitwise<Op>::value;
     using wide_int = typename std::conditional<
         sizeof(T) == 8, typename std::conditional<arith || std::is_unsigned<T>::value, uint64_t, int64_t>::type,
         typename std::conditional<arith || std::is_unsigned<T>::value, uint32_t, int32_t>::type>::type;
@@ -100,8 +111,10 @@ template <typename T, typename Op> __device__ __forceinline__ typename AccOf<T, 
     using A = typename AccOf<T, Op>::type;
     if constexpr (IsCplx<T>::value)
         return A{std::is_same<Op, OpMul>::value ? 1 : 0, 0};
-    else if constexpr (std::is_same<Op, OpAdd>::value)
+    else if constexpr (std::is_same<Op, OpAdd>::value || std::is_same<Op, OpOr>::value || std::is_same<Op, OpXor>::value)
         return A(0);
+    else if constexpr (std::is_same<Op, OpAnd>::value)
+        return (A) ~(A)0;
     else if constexpr (std::is_same<Op, OpMul>::value)
         return A(1);
     else if constexpr (std::is_same<Op, OpMax>::value)
@@ -374,8 +387,17 @@ int launch_op(int op, const void *in, int64_t n, int64_t stride, const void *ini
     case NBH_MUL: return launch<T, OpMul>(in, n, stride, init, out, scratch, s);
     case NBH_MAX: return launch<T, OpMax>(in, n, stride, init, out, scratch, s);
     case NBH_MIN: return launch<T, OpMin>(in, n, stride, init, out, scratch, s);
-    default: return (int)hipErrorInvalidValue;
+    default: break;
     }
+    if constexpr (std::is_integral<T>::value) {
+        switch (op) {
+        case NBH_AND: return launch<T, OpAnd>(in, n, stride, init, out, scratch, s);
+        case NBH_OR: return launch<T, OpOr>(in, n, stride, init, out, scratch, s);
+        case NBH_XOR: return launch<T, OpXor>(in, n, stride, init, out, scratch, s);
+        default: break;
+        }
+    }
+    return (int)hipErrorInvalidValue;
 }
 
 // complex elements: sums and products only (there is no order to take a maximum by)

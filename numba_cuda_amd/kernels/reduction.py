@@ -2,8 +2,8 @@
 
 Drop-in for numba_cuda/numba/cuda/kernels/reduction.py:169-265.  The reference
 JIT-compiles the Python functor into a three-launch tree reduction; here the
-functor is *recognised* as one of the four operators that have hand-written HIP
-kernels (a + b, a * b, max(a, b), min(a, b)) and a single launch of
+functor is *recognised* as one of the operators that have hand-written HIP
+kernels (a + b, a * b, max(a, b), min(a, b), and a & b, a | b, a ^ b on integers) and a single launch of
 nbh_reduce does the work.  Anything else raises NotImplementedError - there is
 no slower path to fall back to.
 """
@@ -41,6 +41,24 @@ class _Sym:
 
     def __rmul__(self, o):
         return self._binary("mul", o, True)
+
+    def __and__(self, o):
+        return self._binary("and", o)
+
+    def __rand__(self, o):
+        return self._binary("and", o, True)
+
+    def __or__(self, o):
+        return self._binary("or", o)
+
+    def __ror__(self, o):
+        return self._binary("or", o, True)
+
+    def __xor__(self, o):
+        return self._binary("xor", o)
+
+    def __rxor__(self, o):
+        return self._binary("xor", o, True)
 
     def _compare(self, opname, other):
         if not isinstance(other, _Sym):
@@ -84,7 +102,10 @@ class _Unrecognised(Exception):
 
 
 _DIRECT = {operator.add: "add", operator.mul: "mul", max: "max", min: "min",
-           np.add: "add", np.multiply: "mul"}
+           np.add: "add", np.multiply: "mul",
+           operator.and_: "and", operator.or_: "or", operator.xor: "xor",
+           np.bitwise_and: "and", np.bitwise_or: "or", np.bitwise_xor: "xor"}
+_ARITHMETIC = ("add", "mul", "and", "or", "xor")
 
 
 def _trace(functor, answer):
@@ -97,7 +118,7 @@ def _trace(functor, answer):
 
 
 def classify_functor(functor):
-    """-> "add" | "mul" | "max" | "min", or NotImplementedError.
+    """-> "add" | "mul" | "max" | "min" | "and" | "or" | "xor", or NotImplementedError.
 
     The functor is run on two recording stand-ins.  `a + b` / `a * b` show up as
     one arithmetic event.  `max(a, b)` / `min(a, b)` and the equivalent
@@ -113,7 +134,7 @@ def classify_functor(functor):
     try:
         name_t, log_t = _trace(functor, True)
         name_f, log_f = _trace(functor, False)
-        if len(log_t) == 1 and log_t == log_f and log_t[0][0] in ("add", "mul"):
+        if len(log_t) == 1 and log_t == log_f and log_t[0][0] in _ARITHMETIC:
             if {log_t[0][1], log_t[0][2]} == {"a", "b"}:
                 verdict = log_t[0][0]
         elif (len(log_t) == 1 and len(log_f) == 1 and log_t[0][0] == "cmp" and log_t == log_f
@@ -128,7 +149,7 @@ def classify_functor(functor):
     except Exception:
         verdict = None
     if verdict is not None:
-        probes = {"add": 8, "mul": 15, "max": 5, "min": 3}
+        probes = {"add": 8, "mul": 15, "max": 5, "min": 3, "and": 1, "or": 7, "xor": 6}
         try:
             ok = functor(3, 5) == probes[verdict] and functor(5, 3) == probes[verdict]
         except Exception:
@@ -136,7 +157,8 @@ def classify_functor(functor):
         if ok:
             return verdict
     raise NotImplementedError(
-        "Reduce supports the binary operators a + b, a * b, max(a, b) and min(a, b); "
+        "Reduce supports the binary operators a + b, a * b, max(a, b), min(a, b) and, for integers, "
+        "a & b, a | b, a ^ b; "
         "%r was not recognised as one of them" % (functor,))
 
 
@@ -167,6 +189,9 @@ class Reduce:
         if dtype.kind == "c" and self._op in ("max", "min"):
             # the reference fails the same way, at compile time: complex numbers are not ordered
             raise TypeError("max / min are not defined for %s" % dtype)
+        if dtype.kind not in "iu" and self._op in ("and", "or", "xor"):
+            # the reference fails at compile time too: no bitwise operators on floating point
+            raise TypeError("bitwise %s is not defined for %s" % (self._op, dtype))
         return code
 
     def __call__(self, arr, size=None, res=None, init=0, stream=0):

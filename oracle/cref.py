@@ -27,6 +27,9 @@ COMPLEX_SUFFIX = {"c64": np.complex64, "c128": np.complex128}
 COMPLEX_OPS = ("add", "mul")
 _SUFFIX_OF = {np.dtype(v): k for k, v in list(SUFFIX.items()) + list(COMPLEX_SUFFIX.items())}
 OPS = ("add", "mul", "max", "min")
+# bitwise functors exist for the integer element types only
+BITWISE_OPS = ("and", "or", "xor")
+INT_SUFFIX = {k: v for k, v in SUFFIX.items() if np.dtype(v).kind in "iu"}
 
 STATE_DTYPE = np.dtype([("s0", np.uint64), ("s1", np.uint64)], align=True)
 
@@ -59,6 +62,10 @@ def lib():
             getattr(L, "orc_xoro_fill_" + kind).argtypes = [_vp, _c_i64, _vp, _c_i64]
         for op in OPS:
             for sfx in SUFFIX:
+                for fam in ("fold", "tree"):
+                    getattr(L, f"orc_{fam}_{op}_{sfx}").argtypes = [_vp, _c_i64, _vp, _vp]
+        for op in BITWISE_OPS:
+            for sfx in INT_SUFFIX:
                 for fam in ("fold", "tree"):
                     getattr(L, f"orc_{fam}_{op}_{sfx}").argtypes = [_vp, _c_i64, _vp, _vp]
         for op in COMPLEX_OPS:

@@ -187,6 +187,11 @@ void orc_xoro_fill_normal_f64(uint64_t *states, int64_t n, double *out, int64_t 
 #define OP_MUL_I(T, U, a, b) ((T)(U)((uint64_t)(U)(a) * (uint64_t)(U)(b)))
 #define OP_ADD_F(T, U, a, b) ((T)((a) + (b)))
 #define OP_MUL_F(T, U, a, b) ((T)((a) * (b)))
+/* bitwise functors (`a & b`, `a | b`, `a ^ b`) on integers: two's complement, like the
+ * reference's LLVM and/or/xor on the element type */
+#define OP_AND_I(T, U, a, b) ((T)(U)((U)(a) & (U)(b)))
+#define OP_OR_I(T, U, a, b) ((T)(U)((U)(a) | (U)(b)))
+#define OP_XOR_I(T, U, a, b) ((T)(U)((U)(a) ^ (U)(b)))
 #define OP_MAX(T, U, a, b) (((b) > (a)) ? (b) : (a))
 #define OP_MIN(T, U, a, b) (((b) < (a)) ? (b) : (a))
 
@@ -297,7 +302,10 @@ void orc_xoro_fill_normal_f64(uint64_t *states, int64_t n, double *out, int64_t 
     DEFINE_REDUCE(add_##sfx, T, U, OP_ADD_I)           \
     DEFINE_REDUCE(mul_##sfx, T, U, OP_MUL_I)           \
     DEFINE_REDUCE(max_##sfx, T, U, OP_MAX)             \
-    DEFINE_REDUCE(min_##sfx, T, U, OP_MIN)
+    DEFINE_REDUCE(min_##sfx, T, U, OP_MIN)             \
+    DEFINE_REDUCE(and_##sfx, T, U, OP_AND_I)           \
+    DEFINE_REDUCE(or_##sfx, T, U, OP_OR_I)             \
+    DEFINE_REDUCE(xor_##sfx, T, U, OP_XOR_I)
 #define DEFINE_REDUCE_FLT(sfx, T)                      \
     DEFINE_REDUCE(add_##sfx, T, T, OP_ADD_F)           \
     DEFINE_REDUCE(mul_##sfx, T, T, OP_MUL_F)           \

@@ -112,6 +112,39 @@ def test_every_operator_and_dtype_against_oracle(op, sfx):
             assert got == cref.tree(op, a, init)
 
 
+@pytest.mark.parametrize("sfx", list(cref.INT_SUFFIX))
+@pytest.mark.parametrize("op", cref.BITWISE_OPS)
+def test_bitwise_operators_on_every_integer_type(op, sfx):
+    """`a & b`, `a | b`, `a ^ b`: bit-exact against the oracle in both association orders
+    (they are associative and commutative, so every order gives the same bits)."""
+    dt = np.dtype(cref.SUFFIX[sfx])
+    functor = {"and": lambda a, b: a & b, "or": lambda a, b: a | b, "xor": lambda a, b: a ^ b}[op]
+    red = cuda.Reduce(functor)
+    rng = np.random.default_rng(abs(hash((op, sfx))) % 2**32)
+    info = np.iinfo(dt)
+    for n in (1, 7, 64, 65, 257, 4096, 300001, 2**21 + 3, 2**24 + 5):
+        _say("reduce", op, sfx, n)
+        a = rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+        if op == "and":                     # keep some bits alive: most elements have most bits set
+            a |= rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+            a |= rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+        elif op == "or":
+            a &= rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+            a &= rng.integers(info.min, info.max, n, dtype=dt, endpoint=True) if n > 64 else a
+        init = {"and": -1 if dt.kind == "i" else info.max, "or": 0, "xor": 5}[op]
+        got = red(a, init=init)
+        assert got.dtype == dt
+        want = {"and": np.bitwise_and, "or": np.bitwise_or, "xor": np.bitwise_xor}[op].reduce(a)
+        if op == "xor":
+            want = want ^ dt.type(5)
+        assert got == want == cref.fold(op, a, init) == cref.tree(op, a, init), (n, got, want)
+    # strided view and a device result slot
+    d = cuda.to_device(a)
+    res = cuda.device_array(1, dt)
+    red(d[::3], res=res, init=init)
+    assert res.copy_to_host()[0] == cref.fold(op, np.ascontiguousarray(a[::3]), init)
+
+
 @pytest.mark.parametrize("dtype", [np.complex64, np.complex128])
 def test_complex_sums_and_products(dtype):
     """Complex elements: sums within 2 n eps sum|x| per component of the exact sums;

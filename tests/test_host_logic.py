@@ -94,6 +94,8 @@ def test_simulator_request_is_refused(monkeypatch):
     (lambda a, b: b if b >= a else a, "max"), (lambda a, b: b if a < b else a, "max"),
     (lambda a, b: min(a, b), "min"), (min, "min"), (lambda a, b: a if a < b else b, "min"),
     (lambda a, b: b if a > b else a, "min"),
+    (lambda a, b: a & b, "and"), (lambda a, b: b & a, "and"), (operator.and_, "and"), (np.bitwise_and, "and"),
+    (lambda a, b: a | b, "or"), (operator.or_, "or"), (lambda a, b: a ^ b, "xor"), (np.bitwise_xor, "xor"),
 ])
 def test_classify_functor(functor, want):
     assert classify_functor(functor) == want
@@ -102,6 +104,7 @@ def test_classify_functor(functor, want):
 @pytest.mark.parametrize("functor", [
     lambda a, b: a - b, lambda a, b: a + b + a, lambda a, b: a, lambda a, b: a + 1,
     lambda a, b: a / b, lambda a, b: 8, lambda a, b: a * a, lambda a, b: a if a else b,
+    lambda a, b: a & 1, lambda a, b: (a ^ b) ^ a, lambda a, b: a << b,
 ])
 def test_unrecognised_functors_raise(functor):
     with pytest.raises(NotImplementedError, match="a \\+ b, a \\* b, max"):

@@ -135,6 +135,25 @@ def test_all_ops_all_dtypes_brute_force(op, sfx):
             assert int(cref.fold(op, a, init)) == acc
 
 
+@pytest.mark.parametrize("sfx", list(cref.INT_SUFFIX))
+@pytest.mark.parametrize("op", cref.BITWISE_OPS)
+def test_bitwise_ops_against_numpy(op, sfx):
+    """and / or / xor are associative and commutative: both orders of the oracle must give
+    NumPy's left-to-right result, bit for bit, for every integer type."""
+    dt = np.dtype(cref.SUFFIX[sfx])
+    info = np.iinfo(dt)
+    ufunc = {"and": np.bitwise_and, "or": np.bitwise_or, "xor": np.bitwise_xor}[op]
+    rng = np.random.default_rng(abs(hash((op, sfx))) % 2**32)
+    for n in (1, 2, 31, 32, 33, 127, 128, 129, 4097, 70001):
+        a = rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+        if op == "and":
+            a |= rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+        for init in (0, 5, info.max, info.min):
+            want = ufunc(ufunc.reduce(a), dt.type(init))
+            assert cref.fold(op, a, init) == want
+            assert cref.tree(op, a, init) == want
+
+
 def test_minmax_follow_python_semantics_for_nan_and_signed_zero():
     # cpython/builtins.py:224-269: max(a, b) = b if b > a else a
     a = np.array([np.nan, 1.0, 2.0], np.float64)
