@@ -183,6 +183,13 @@ class Reduce:
         self._codes = {}    # dtype -> element code, filled once the pairing with the operator is checked
 
     def _element_code(self, dtype):
+        if dtype == _BOOL:
+            # one byte holding 0 or 1: and / or / xor / max / min of those are again 0 or 1,
+            # so the uint8 kernels do (sums and products of booleans are integers in the
+            # reference and are not offered here)
+            if self._op in ("add", "mul"):
+                raise NotImplementedError("Reduce does not add or multiply booleans; use a & b, a | b, a ^ b, max or min")
+            return _DTYPE_CODE[np.dtype(np.uint8)]
         code = _DTYPE_CODE.get(dtype)
         if code is None:
             raise NotImplementedError("Reduce does not support dtype %s" % dtype)
@@ -246,6 +253,7 @@ class Reduce:
 
 
 _DTYPE_CODE = {np.dtype(name): code for name, code in _lib.DTYPE_CODES.items()}
+_BOOL = np.dtype(np.bool_)
 
 # host copies of `init` values, one element each, kept alive for the process:
 # (dtype, init) -> (array, address).  nbh_reduce reads the value during the call.

@@ -145,6 +145,27 @@ def test_bitwise_operators_on_every_integer_type(op, sfx):
     assert res.copy_to_host()[0] == cref.fold(op, np.ascontiguousarray(a[::3]), init)
 
 
+def test_boolean_arrays_any_all_parity():
+    """`a | b`, `a & b`, `a ^ b`, max and min of booleans: any, all, parity, as booleans."""
+    rng = np.random.default_rng(8)
+    any_, all_, par = (cuda.Reduce(lambda a, b: a | b), cuda.Reduce(lambda a, b: a & b),
+                       cuda.Reduce(lambda a, b: a ^ b))
+    mx, mn = cuda.Reduce(lambda a, b: max(a, b)), cuda.Reduce(lambda a, b: min(a, b))
+    for n in (1, 2, 63, 64, 65, 5000, 300001, 2**24 + 5):
+        for p in (0.0, 1.0, 0.5, 1.0 / n, 1.0 - 1.0 / n):
+            a = rng.random(n) < p
+            _say("bool reduce", n, p)
+            got = [any_(a, init=False), all_(a, init=True), par(a, init=False), mx(a, init=False), mn(a, init=True)]
+            assert all(g.dtype == np.bool_ for g in got)
+            assert got == [a.any(), a.all(), bool(a.sum() & 1), a.any(), a.all()], (n, p, got)
+    d = cuda.to_device(a)
+    res = cuda.device_array(1, np.bool_)
+    any_(d[::2], res=res)
+    assert res.copy_to_host()[0] == a[::2].any()
+    with pytest.raises(NotImplementedError, match="booleans"):
+        cuda.Reduce(lambda a, b: a + b)(a)
+
+
 @pytest.mark.parametrize("dtype", [np.complex64, np.complex128])
 def test_complex_sums_and_products(dtype):
     """Complex elements: sums within 2 n eps sum|x| per component of the exact sums;

@@ -84,6 +84,8 @@ def test_reduce_host_side_contract(fake_gpu):
         red(np.zeros(4, np.float16))
     with pytest.raises(TypeError, match="not defined for complex64"):
         cuda.reduce(lambda a, b: max(a, b))(np.zeros(4, np.complex64))
+    with pytest.raises(NotImplementedError, match="does not add or multiply booleans"):
+        red(np.zeros(4, np.bool_))
     with pytest.raises(TypeError, match="bitwise xor is not defined for float32"):
         cuda.reduce(lambda a, b: a ^ b)(np.zeros(4, np.float32))
 
