@@ -172,6 +172,27 @@ size_t nbh_reduce_scratch_bytes(void);
 int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                void *scratch, size_t scratch_bytes, nbh_stream_t stream);
 
+/* nbh_reduce for callers that cannot allocate device memory: code under stream (graph)
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
+ * in the reference (whose Reduce.__call__ allocates its partials on every call,
+ * kernels/reduction.py:242).  Same arguments, kernels and results as nbh_reduce, minus
+ * the scratch buffer: ticket and partials live in a 33 KiB array that is part of the
+ * library's code object, one copy per device, held until the process ends.  The call
+ * makes no hipMalloc / hipFree / hipHostMalloc and no allocating library call (host side:
+ * one map node the first time a stream is seen while the pooling manager is in use).
+ * The address of the array is looked up on the first call on each device: make that call
+ * outside stream capture.
+ *   - n above NBH_REDUCE_NOALLOC_MAX_ITEMS is refused with hipErrorInvalidValue before
+ *     anything is launched
+ *   - every call on a device shares that device's array: calls that may overlap in time
+ *     (different streams, different host threads) race and give wrong results; callers
+ *     that need overlap bring one scratch buffer per stream to nbh_reduce instead
+ *   - the array starts zeroed and each call leaves its ticket at zero again; the partials
+ *     keep the last call's values and are overwritten before they are read */
+#define NBH_REDUCE_NOALLOC_MAX_ITEMS ((int64_t)1 << 36)
+int nbh_reduce_noalloc(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init,
+                       void *out, nbh_stream_t stream);
+
 /* ---- transpose ------------------------------------------------------------ */
 
 /* kernels/transpose.py:10-65 transpose(a, b): out[j, i] = in[i, j] for a

@@ -36,7 +36,9 @@
 // HBM roofline: n * itemsize bytes are read once; nothing else of size is moved.
 #include "common.h"
 
+#include <atomic>
 #include <limits>
+#include <mutex>
 #include <type_traits>
 
 namespace {
@@ -444,3 +446,53 @@ int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, 
 }
 
 }  // extern "C"
+
+// ---- the same reduction for callers that cannot allocate ------------------------------
+// Ticket and partials live in an array inside the code object: every device the library
+// runs on holds its own copy, at its own address, from the moment the code object is
+// loaded there until the process ends.  The array's name is a host-side stand-in; the
+// address kernels can use is looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_static_scratch[kMaxDevices];  // device address of `scratch`, per device
+std::mutex g_static_mu;
+
+// Address of the current device's copy of `scratch`.
+int static_scratch(void **out)
+{
+    int dev = -1;
+    NBH_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices)
+        return (int)hipErrorInvalidDevice;
+    void *p = g_static_scratch[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(g_static_mu);
+        p = g_static_scratch[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            NBH_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            if (!p)
+                return (int)hipErrorInvalidSymbol;
+            // the array is zero when the code object is loaded, and every reduction hands
+            // the ticket back at zero: nothing to clear here
+            g_static_scratch[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int nbh_reduce_noalloc(int op, int dtype, const void *in, int64_t n, int64_t in_stride,
+                                  const void *init, void *out, nbh_stream_t stream)
+{
+    if (n > NBH_REDUCE_NOALLOC_MAX_ITEMS)
+        return (int)hipErrorInvalidValue;  // stated limit of this entry point; nothing is launched
+    void *ptr = nullptr;
+    if (int rc = static_scratch(&ptr))
+        return rc;
+    return nbh_reduce(op, dtype, in, n, in_stride, init, out, ptr, kScratchBytes, stream);
+}
