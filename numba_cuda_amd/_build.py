@@ -62,12 +62,7 @@ def find_hipcc():
     raise RuntimeError("hipcc not found (set HIPCC or install ROCm under /opt/rocm)")
 
 
-def build(verbose=False):
-    """Compile every HIP source into numba_cuda_amd/libnbhip.so; returns its path."""
-    cmd = [find_hipcc()] + HIPCC_FLAGS + ["-I", INCLUDE_DIR, "-I", SRC_DIR]
-    cmd += [os.path.join(SRC_DIR, s) for s in SOURCES]
-    tmp = LIB_PATH + ".tmp"
-    cmd += ["-o", tmp]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -78,10 +73,36 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
+
+
+def build(verbose=False, only=None):
+    """Compile every HIP source (or just the names in `only`, reusing the other object
+    files) and link numba_cuda_amd/libnbhip.so; returns its path.  Sources compile side
+    by side, one hipcc process each."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    hipcc = find_hipcc()
+    obj_dir = os.path.join(PKG_DIR, "_obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    objects, jobs = [], []
+    for src in SOURCES:
+        obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+        objects.append(obj)
+        if only is None or src in only or not os.path.exists(obj):
+            jobs.append([hipcc] + compile_flags + ["-I", INCLUDE_DIR, "-I", SRC_DIR, "-c",
+                                                   os.path.join(SRC_DIR, src), "-o", obj])
+    workers = max(1, min(len(jobs), os.cpu_count() or 1, 8))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        for _ in pool.map(lambda cmd: _run(cmd, verbose), jobs):
+            pass
+    tmp = LIB_PATH + ".tmp"
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", tmp], verbose)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 
 
 if __name__ == "__main__":
     print(build_hostbuf(verbose="-v" in sys.argv))
-    print(build(verbose="-v" in sys.argv))
+    names = [a for a in sys.argv[1:] if a.endswith(".hip")]
+    print(build(verbose="-v" in sys.argv, only=names or None))
