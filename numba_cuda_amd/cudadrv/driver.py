@@ -1,20 +1,21 @@
 """HIP driver layer: devices, contexts, memory objects, streams, events, copies.
 
-Python owns every lifetime here, as in the reference
-(numba_cuda/numba/cuda/cudadrv/driver.py): device memory is a `MemoryPointer`
-whose finalizer does not free but *queues* the free in the context's
-`_PendingDeallocs`, so that garbage collection never turns into a device-wide
-synchronisation in the middle of asynchronous work.  Underneath there is no
-driver binding, only the C entry points of libnbhip.so (include/nbhip.h).
-
-HIP has one implicit primary context per device, so `Context` is a per-device
-bookkeeping object (memory manager, pending frees, reduction scratch) rather
+The public names and their behaviour follow numba_cuda/numba/cuda/cudadrv/driver.py
+of the reference (each class cites the lines it stands in for), so that code written
+against `numba.cuda.cudadrv.driver` keeps working.  What is underneath is different:
+there is no driver binding, only the C entry points of libnbhip.so (include/nbhip.h),
+and HIP has one implicit primary context per device, so `Context` is a per-device
+bookkeeping object (memory manager, releases that wait, reduction scratch) rather
 than a driver handle.
+
+Lifetimes are owned here, in Python.  Device memory is a `MemoryPointer`; when its
+last owner goes away the raw free is not executed but parked in the context's queue
+of waiting releases (`_PendingDeallocs`) and carried out in batches, so that garbage
+collection never turns into a device-wide synchronisation in the middle of
+asynchronous work.
 """
 
-import contextlib
 import ctypes
-import functools
 import importlib
 import logging
 import os
@@ -22,8 +23,8 @@ import sys
 import threading
 import weakref
 from abc import ABCMeta, abstractmethod
-from collections import deque, namedtuple
-from ctypes import c_int, c_size_t, c_void_p, byref
+from collections import namedtuple
+from ctypes import byref, c_int, c_size_t, c_void_p
 
 import numpy as np
 
@@ -40,18 +41,19 @@ from numba_cuda_amd.core.errors import CudaDriverError, CudaSupportError  # noqa
 
 
 def make_logger():
-    logger = logging.getLogger(__name__)
-    lvl = str(config.CUDA_LOG_LEVEL).upper()
-    lvl = getattr(logging, lvl, None)
-    if not isinstance(lvl, int):
-        logger.addHandler(logging.NullHandler())
+    """Logger of this module.  NUMBA_CUDA_LOG_LEVEL names a level of the logging
+    module; with anything else the logger stays silent."""
+    log = logging.getLogger(__name__)
+    level = getattr(logging, str(config.CUDA_LOG_LEVEL).upper(), None)
+    if isinstance(level, int):
+        log.setLevel(level)
+        if not log.handlers:
+            to_stderr = logging.StreamHandler(sys.stderr)
+            to_stderr.setFormatter(logging.Formatter("== HIP [%(relativeCreated)d] %(levelname)5s -- %(message)s"))
+            log.addHandler(to_stderr)
     else:
-        logger.setLevel(lvl)
-        if not logger.handlers:
-            handler = logging.StreamHandler(sys.stderr)
-            handler.setFormatter(logging.Formatter("== HIP [%(relativeCreated)d] %(levelname)5s -- %(message)s"))
-            logger.addHandler(handler)
-    return logger
+        log.addHandler(logging.NullHandler())
+    return log
 
 
 _logger = make_logger()
@@ -59,15 +61,15 @@ _logger = make_logger()
 
 class CudaAPIError(CudaDriverError):
     """A libnbhip / HIP call returned a non-zero hipError_t (reference:
-    driver.py:147-154; same name so that user except-clauses keep working)."""
+    driver.py:147-154; same name so that user except-clauses keep working).
+    `code` is the hipError_t, `msg` names the call and the error."""
 
     def __init__(self, code, msg):
-        self.code = code
-        self.msg = msg
         super().__init__(code, msg)
+        self.code, self.msg = code, msg
 
     def __str__(self):
-        return "[%s] %s" % (self.code, self.msg)
+        return "[{}] {}".format(self.code, self.msg)
 
 
 HipAPIError = CudaAPIError
@@ -89,31 +91,34 @@ class Driver:
             obj.initialization_error = None
             obj.pid = None
             obj._lock = threading.Lock()
+            obj._devices = {}
             cls._singleton = obj
         return cls._singleton
 
-    def ensure_initialized(self):
-        if self.is_initialized:
-            if self.initialization_error is not None:
-                raise CudaSupportError("Error at driver init: %s" % self.initialization_error)
-            return
-        with self._lock:
-            if self.is_initialized:
-                return
-            self.is_initialized = True
-            if config.DISABLE_CUDA:
-                self.initialization_error = "GPU support disabled by NUMBA_DISABLE_CUDA=1"
-            elif config.ENABLE_CUDASIM:
-                self.initialization_error = ("NUMBA_ENABLE_CUDASIM=1 asks for the CPU simulator, "
-                                             "which this GPU-only package does not provide")
-            else:
-                try:
-                    self.lib = _lib.load()
-                    self.pid = os.getpid()
-                except OSError as e:
-                    self.initialization_error = str(e)
+    def _refuse_if_broken(self):
         if self.initialization_error is not None:
             raise CudaSupportError("Error at driver init: %s" % self.initialization_error)
+
+    def ensure_initialized(self):
+        if not self.is_initialized:
+            with self._lock:
+                if not self.is_initialized:
+                    self._load()
+                    self.is_initialized = True
+        self._refuse_if_broken()
+
+    def _load(self):
+        if config.DISABLE_CUDA:
+            self.initialization_error = "GPU support disabled by NUMBA_DISABLE_CUDA=1"
+        elif config.ENABLE_CUDASIM:
+            self.initialization_error = ("NUMBA_ENABLE_CUDASIM=1 asks for the CPU simulator, "
+                                         "which this GPU-only package does not provide")
+        else:
+            try:
+                self.lib = _lib.load()
+                self.pid = os.getpid()
+            except OSError as e:
+                self.initialization_error = str(e)
 
     @property
     def is_available(self):
@@ -128,24 +133,33 @@ class Driver:
         return name.decode() if name else "hipError_%d" % code
 
     def check(self, fname, code):
-        if code != _lib.HIP_SUCCESS:
-            if self.pid is not None and os.getpid() != self.pid:
-                raise CudaDriverError("HIP initialized before forking")
-            raise CudaAPIError(code, "Call to %s results in %s" % (fname, self._error_name(code)))
+        """Raise for a non-zero status of the call named `fname`."""
+        if code == _lib.HIP_SUCCESS:
+            return
+        if self.pid is not None and os.getpid() != self.pid:
+            # a forked child inherits a runtime it cannot use
+            raise CudaDriverError("HIP initialized before forking")
+        raise CudaAPIError(code, "Call to %s results in %s" % (fname, self._error_name(code)))
 
     def __getattr__(self, fname):
+        # first use of an entry point: build its checked wrapper and keep it
         if not fname.startswith("nbh_"):
             raise AttributeError(fname)
         self.ensure_initialized()
-        cfn = getattr(self.lib, fname)
+        entry = getattr(self.lib, fname)
+        check = self.check
 
         def checked(*args):
-            if config.CUDA_LOG_API_ARGS:
-                _logger.debug("call driver api: %s%r", fname, args)
-            else:
-                _logger.debug("call driver api: %s", fname)
-            self.check(fname, cfn(*args))
+            if _logger.isEnabledFor(logging.DEBUG):
+                if config.CUDA_LOG_API_ARGS:
+                    _logger.debug("call driver api: %s%r", fname, args)
+                else:
+                    _logger.debug("call driver api: %s", fname)
+            status = entry(*args)
+            if status:
+                check(fname, status)
 
+        checked.__name__ = fname
         setattr(self, fname, checked)
         return checked
 
@@ -155,11 +169,14 @@ class Driver:
         self.nbh_device_count(byref(n))
         return n.value
 
-    @functools.lru_cache(maxsize=None)
     def get_device(self, devnum=0):
-        if not 0 <= devnum < self.get_device_count():
-            raise CudaAPIError(101, "Call to hipSetDevice results in hipErrorInvalidDevice")
-        return Device(devnum)
+        dev = self._devices.get(devnum)
+        if dev is None:
+            if not 0 <= devnum < self.get_device_count():
+                raise CudaAPIError(101, "Call to hipSetDevice results in hipErrorInvalidDevice")
+            with self._lock:
+                dev = self._devices.setdefault(devnum, Device(devnum))
+        return dev
 
     def list_devices(self):
         return [self.get_device(i) for i in range(self.get_device_count())]
@@ -224,79 +241,165 @@ class Device:
     def __repr__(self):
         return "<HIP device %d '%s'>" % (self.id, self.name)
 
-    def __hash__(self):
-        return hash(self.id)
-
     def __eq__(self, other):
-        return isinstance(other, Device) and self.id == other.id
+        return isinstance(other, Device) and other.id == self.id
+
+    def __hash__(self):
+        return hash(("hip-device", self.id))
 
 
 # --------------------------------------------------------------------------------
-# Pending deallocations
+# Releases that wait
 # --------------------------------------------------------------------------------
 
-class _SizeNotSet(int):
-    """Stand-in size of a resource whose footprint is unknown (counts as 0)."""
+class _Hold:
+    """`with queue.disable():` - one more reason not to flush while inside."""
 
-    def __new__(cls, *args, **kwargs):
-        return super().__new__(cls, 0)
+    __slots__ = ("_queue",)
 
-    def __str__(self):
-        return "?"
+    def __init__(self, queue):
+        self._queue = queue
 
+    def __enter__(self):
+        with self._queue._lock:
+            self._queue._holds += 1
+        return self._queue
 
-_SizeNotSet = _SizeNotSet()
+    def __exit__(self, exc_type, exc, tb):
+        with self._queue._lock:
+            self._queue._holds -= 1
+        return False
 
 
 class _PendingDeallocs:
-    """Queue of (destructor, handle, size) to run later (reference :975-1045).
+    """Releases (`release(handle)` calls) parked until there are enough of them
+    (reference :975-1045; the counts and thresholds are the ones its
+    tests/cudadrv/test_deallocations.py pins).
 
-    Flushed when more than CUDA_DEALLOCS_COUNT entries or more than
-    CUDA_DEALLOCS_RATIO * capacity bytes are waiting, on out-of-memory, and on
-    reset.  `disable()` is a nestable context manager that holds flushing off.
-    """
+    `add_item` parks one; the whole batch is carried out as soon as more than
+    config.CUDA_DEALLOCS_COUNT entries, or more than config.CUDA_DEALLOCS_RATIO of
+    `memory_capacity` bytes, are waiting - and by `clear()`, which the allocator
+    calls when the device runs out of memory and the context calls on reset.
+    Inside `with queue.disable():` (nestable) nothing is carried out at all.
 
-    def __init__(self, capacity=_SizeNotSet):
-        self._cons = deque()
-        self._disable_count = 0
-        self._size = 0
+    Finalizers run on whatever thread drops the last reference, so the queue is
+    guarded by a lock; the batch is taken out of the queue before the first release
+    runs, which makes a release that parks further entries harmless.
+
+    `memory_capacity` is None until the memory manager has asked the device; the
+    byte threshold is 0 until then."""
+
+    def __init__(self, capacity=None):
         self.memory_capacity = capacity
+        self._lock = threading.RLock()
+        self._waiting = []          # (release, handle, bytes or None)
+        self._waiting_bytes = 0
+        self._holds = 0
 
     @property
-    def _max_pending_bytes(self):
-        return int(self.memory_capacity * config.CUDA_DEALLOCS_RATIO)
+    def byte_budget(self):
+        """Bytes that may wait before a flush."""
+        if self.memory_capacity is None:
+            return 0
+        return int(config.CUDA_DEALLOCS_RATIO * self.memory_capacity)
 
-    def add_item(self, dtor, handle, size=_SizeNotSet):
-        _logger.info("add pending dealloc: %s %s bytes", getattr(dtor, "__name__", dtor), size)
-        self._cons.append((dtor, handle, size))
-        self._size += int(size)
-        if len(self._cons) > config.CUDA_DEALLOCS_COUNT or self._size > self._max_pending_bytes:
+    @property
+    def pending_bytes(self):
+        """Bytes (of entries with a known size) waiting now."""
+        return self._waiting_bytes
+
+    # the reference's own test-suite reads these two private names
+    _max_pending_bytes = byte_budget
+    _size = pending_bytes
+
+    def add_item(self, release, handle, size=None):
+        """Park `release(handle)`; `size` is the footprint in bytes when known."""
+        _logger.info("park release: %s, %s bytes", _name_of(release), "?" if size is None else size)
+        with self._lock:
+            self._waiting.append((release, handle, size))
+            if size is not None:
+                self._waiting_bytes += int(size)
+            full = (len(self._waiting) > config.CUDA_DEALLOCS_COUNT
+                    or self._waiting_bytes > self.byte_budget)
+        if full:
             self.clear()
 
     def clear(self):
-        if self.is_disabled:
-            return
-        while self._cons:
-            dtor, handle, size = self._cons.popleft()
-            _logger.info("dealloc: %s %s bytes", getattr(dtor, "__name__", dtor), size)
-            dtor(handle)
-        self._size = 0
-
-    @contextlib.contextmanager
-    def disable(self):
-        self._disable_count += 1
+        """Carry out everything that waits - unless flushing is held off."""
+        with self._lock:
+            if self._holds:
+                return
+            batch, self._waiting = self._waiting, []
+            self._waiting_bytes = 0
+        done = 0
         try:
-            yield
+            for release, handle, size in batch:
+                _logger.info("release: %s, %s bytes", _name_of(release), "?" if size is None else size)
+                done += 1
+                release(handle)
         finally:
-            self._disable_count -= 1
-            assert self._disable_count >= 0
+            if done < len(batch):       # a release raised: the rest goes back to the front
+                with self._lock:
+                    rest = batch[done:]
+                    self._waiting[:0] = rest
+                    self._waiting_bytes += sum(int(s) for _, _, s in rest if s is not None)
+
+    def disable(self):
+        """Context manager: no flushing inside (the queue only grows)."""
+        return _Hold(self)
 
     @property
     def is_disabled(self):
-        return self._disable_count > 0
+        return self._holds > 0
 
     def __len__(self):
-        return len(self._cons)
+        return len(self._waiting)
+
+
+def _name_of(fn):
+    return getattr(fn, "__name__", None) or repr(fn)
+
+
+class _Release:
+    """Finalizer of one tracked allocation: take it out of the manager's table of
+    live allocations and hand the raw free to the queue of waiting releases - or,
+    with no queue, carry it out on the spot (reference :1316-1371 has three
+    closures for this).  Built from the tables themselves rather than the manager, so
+    that the finalizer does not keep the manager (and its context) alive."""
+
+    __slots__ = ("table", "key", "queue", "raw_free", "address", "nbytes")
+
+    def __init__(self, raw_free, address, nbytes=None, table=None, key=None, queue=None):
+        self.raw_free, self.address, self.nbytes = raw_free, address, nbytes
+        self.table, self.key, self.queue = table, key, queue
+
+    def __call__(self):
+        if self.table is not None:
+            self.table.pop(self.key, None)
+        if self.queue is None:
+            self.raw_free(self.address)
+        else:
+            self.queue.add_item(self.raw_free, self.address, self.nbytes)
+
+
+def _free_device(ptr):
+    driver.nbh_free(ptr)
+
+
+def _free_host(ptr):
+    driver.nbh_host_free(ptr)
+
+
+def _unregister_host(ptr):
+    driver.nbh_host_unregister(ptr)
+
+
+def _destroy_stream(handle):
+    driver.nbh_stream_destroy(handle)
+
+
+def _destroy_event(handle):
+    driver.nbh_event_destroy(handle)
 
 
 MemoryInfo = namedtuple("MemoryInfo", "free,total")
@@ -306,11 +409,18 @@ MemoryInfo = namedtuple("MemoryInfo", "free,total")
 # Memory managers (the EMM plugin interface of the reference, :589-957)
 # --------------------------------------------------------------------------------
 
+_SUPPORTED_EMM_INTERFACE_VERSION = 1
+
+
 class BaseCUDAMemoryManager(metaclass=ABCMeta):
+    """What an external memory manager has to provide.  One instance is made per
+    context, with the context passed as a keyword."""
+
     def __init__(self, *args, **kwargs):
-        if "context" not in kwargs:
-            raise RuntimeError("Memory manager requires a context")
-        self.context = kwargs.pop("context")
+        try:
+            self.context = kwargs.pop("context")
+        except KeyError:
+            raise RuntimeError("Memory manager requires a context") from None
 
     @abstractmethod
     def memalloc(self, size):
@@ -352,7 +462,10 @@ class BaseCUDAMemoryManager(metaclass=ABCMeta):
 
 class HostOnlyCUDAMemoryManager(BaseCUDAMemoryManager):
     """Host-side allocations plus the bookkeeping every manager needs; plugins
-    that only care about device memory derive from this (reference :705-872)."""
+    that only care about device memory derive from this (reference :705-872).
+
+    `allocations` maps the address of every live tracked allocation to its memory
+    object, `deallocations` is the queue of releases that wait."""
 
     def __init__(self, *args, **kwargs):
         super().__init__(*args, **kwargs)
@@ -360,70 +473,75 @@ class HostOnlyCUDAMemoryManager(BaseCUDAMemoryManager):
         self.deallocations = _PendingDeallocs()
 
     def _attempt_allocation(self, allocator):
-        """Run `allocator`; on out-of-memory flush pending frees and retry once."""
-        try:
-            return allocator()
-        except CudaAPIError as e:
-            if e.code != _lib.HIP_ERROR_OUT_OF_MEMORY:
-                raise
-            self.deallocations.clear()
-            return allocator()
+        """Result of `allocator()`.  If the device is out of memory, everything
+        that waits to be released is released and the allocation tried once more."""
+        for last_try in (False, True):
+            try:
+                return allocator()
+            except CudaAPIError as e:
+                if last_try or e.code != _lib.HIP_ERROR_OUT_OF_MEMORY:
+                    raise
+                self.deallocations.clear()
+
+    def _track(self, mem, address):
+        self.allocations[address] = mem
+        return mem.own()
+
+    def _context_proxy(self):
+        return weakref.proxy(self.context)
 
     def memhostalloc(self, size, mapped=False, portable=False, wc=False):
         flags = (1 if portable else 0) | (2 if mapped else 0) | (4 if wc else 0)
 
-        def allocator():
-            p = c_void_p()
-            driver.nbh_host_alloc(byref(p), size, flags)
-            return p.value or 0
+        def allocate():
+            out = c_void_p()
+            driver.nbh_host_alloc(byref(out), size, flags)
+            return out.value or 0
 
-        pointer = self._attempt_allocation(allocator) if mapped else allocator()
-        finalizer = _hostalloc_finalizer(self, pointer, pointer, size, mapped)
-        ctx = weakref.proxy(self.context)
-        if mapped:
-            mem = MappedMemory(ctx, pointer, size, finalizer=finalizer)
-            self.allocations[pointer] = mem
-            return mem.own()
-        return PinnedMemory(ctx, pointer, size, finalizer=finalizer)
+        if not mapped:
+            # plain page-locked memory: not in the table, footprint on the device unknown
+            address = allocate()
+            return PinnedMemory(self._context_proxy(), address, size,
+                                finalizer=_Release(_free_host, address, queue=self.deallocations))
+        address = self._attempt_allocation(allocate)
+        on_release = _Release(_free_host, address, size, self.allocations, address, self.deallocations)
+        return self._track(MappedMemory(self._context_proxy(), address, size, finalizer=on_release), address)
 
     def mempin(self, owner, pointer, size, mapped=False):
-        flags = 2 if mapped else 0
+        def register():
+            driver.nbh_host_register(pointer, size, 2 if mapped else 0)
 
-        def allocator():
-            driver.nbh_host_register(pointer, size, flags)
-
-        if mapped:
-            self._attempt_allocation(allocator)
-        else:
-            allocator()
-        finalizer = _pin_finalizer(self, pointer, pointer, mapped)
-        ctx = weakref.proxy(self.context)
-        if mapped:
-            mem = MappedMemory(ctx, pointer, size, owner=owner, finalizer=finalizer)
-            self.allocations[pointer] = mem
-            return mem.own()
-        return PinnedMemory(ctx, pointer, size, owner=owner, finalizer=finalizer)
+        # Page-locking is undone the moment the object dies, not queued: the same
+        # host buffer may be pinned again right away (`with cuda.pinned(a): ...` twice).
+        if not mapped:
+            register()
+            return PinnedMemory(self._context_proxy(), pointer, size, owner=owner,
+                                finalizer=_Release(_unregister_host, pointer))
+        self._attempt_allocation(register)
+        on_release = _Release(_unregister_host, pointer, table=self.allocations, key=pointer)
+        mem = MappedMemory(self._context_proxy(), pointer, size, owner=owner, finalizer=on_release)
+        return self._track(mem, pointer)
 
     def memallocmanaged(self, size, attach_global):
-        def allocator():
-            p = c_void_p()
-            driver.nbh_malloc_managed(byref(p), size, 1 if attach_global else 0)
-            return p.value or 0
+        def allocate():
+            out = c_void_p()
+            driver.nbh_malloc_managed(byref(out), size, 1 if attach_global else 0)
+            return out.value or 0
 
-        ptr = self._attempt_allocation(allocator)
-        finalizer = _alloc_finalizer(self, ptr, ptr, size)
-        mem = ManagedMemory(weakref.proxy(self.context), ptr, size, finalizer=finalizer)
-        self.allocations[ptr] = mem
-        return mem.own()
+        address = self._attempt_allocation(allocate)
+        on_release = _Release(_free_device, address, size, self.allocations, address, self.deallocations)
+        return self._track(ManagedMemory(self._context_proxy(), address, size, finalizer=on_release), address)
 
     def reset(self):
-        self.allocations.clear()
+        """Forget every tracked allocation (objects nobody else holds are finalized,
+        which parks their frees), then carry out everything that waits."""
+        tracked = self.allocations
+        tracked.clear()
         self.deallocations.clear()
 
-    @contextlib.contextmanager
     def defer_cleanup(self):
-        with self.deallocations.disable():
-            yield
+        """Context manager: no waiting release is carried out inside."""
+        return self.deallocations.disable()
 
 
 class GetIpcHandleMixin:
@@ -444,79 +562,128 @@ class GetIpcHandleMixin:
 
 
 class NumbaCUDAMemoryManager(GetIpcHandleMixin, HostOnlyCUDAMemoryManager):
-    """Default manager: hipMalloc per allocation, deferred hipFree (reference
-    :892-921)."""
+    """The manager used unless another is plugged in: one hipMalloc per allocation,
+    hipFree through the queue of waiting releases (reference :885-915)."""
+
+    interface_version = _SUPPORTED_EMM_INTERFACE_VERSION
 
     def initialize(self):
-        if self.deallocations.memory_capacity == _SizeNotSet:
-            self.deallocations.memory_capacity = self.get_memory_info().total
+        queue = self.deallocations
+        if queue.memory_capacity is None:       # first use: now the device can be asked
+            queue.memory_capacity = self.get_memory_info().total
 
     def memalloc(self, size):
-        def allocator():
-            p = c_void_p()
-            driver.nbh_malloc(byref(p), size)
-            return p.value or 0
+        def allocate():
+            out = c_void_p()
+            driver.nbh_malloc(byref(out), size)
+            return out.value or 0
 
-        ptr = self._attempt_allocation(allocator)
-        finalizer = _alloc_finalizer(self, ptr, ptr, size)
-        mem = AutoFreePointer(weakref.proxy(self.context), ptr, size, finalizer=finalizer)
-        self.allocations[ptr] = mem
-        return mem.own()
+        address = self._attempt_allocation(allocate)
+        on_release = _Release(_free_device, address, size, self.allocations, address, self.deallocations)
+        return self._track(AutoFreePointer(self._context_proxy(), address, size, finalizer=on_release), address)
 
     def get_memory_info(self):
         free, total = c_size_t(), c_size_t()
         driver.nbh_mem_info(byref(free), byref(total))
         return MemoryInfo(free=free.value, total=total.value)
 
-    @property
-    def interface_version(self):
-        return _SUPPORTED_EMM_INTERFACE_VERSION
 
-
-_SUPPORTED_EMM_INTERFACE_VERSION = 1
+# the class new contexts instantiate; None until the first context (or set_memory_manager)
 _memory_manager = None
-
-
-def _ensure_memory_manager():
-    global _memory_manager
-    if _memory_manager:
-        return
-    if config.CUDA_MEMORY_MANAGER == "default":
-        _memory_manager = NumbaCUDAMemoryManager
-        return
-    try:
-        mgr_module = importlib.import_module(config.CUDA_MEMORY_MANAGER)
-        set_memory_manager(mgr_module._numba_memory_manager)
-    except Exception:
-        raise RuntimeError("Failed to use memory manager from %s" % config.CUDA_MEMORY_MANAGER)
 
 
 def set_memory_manager(mm_plugin):
     """Use an External Memory Management plugin class for all later contexts."""
     global _memory_manager
-    iv = mm_plugin(context=None).interface_version
-    if iv != _SUPPORTED_EMM_INTERFACE_VERSION:
+    found = mm_plugin(context=None).interface_version
+    if found != _SUPPORTED_EMM_INTERFACE_VERSION:
         raise RuntimeError("EMM Plugin interface has version %d - version %d required"
-                           % (iv, _SUPPORTED_EMM_INTERFACE_VERSION))
+                           % (found, _SUPPORTED_EMM_INTERFACE_VERSION))
     _memory_manager = mm_plugin
+
+
+def _ensure_memory_manager():
+    """Settle which manager class contexts use: one set by hand wins, then the
+    module NUMBA_CUDA_MEMORY_MANAGER names (its `_numba_memory_manager`), then the
+    built-in one."""
+    global _memory_manager
+    if _memory_manager is not None:
+        return
+    wanted = config.CUDA_MEMORY_MANAGER
+    if wanted == "default":
+        _memory_manager = NumbaCUDAMemoryManager
+        return
+    try:
+        set_memory_manager(importlib.import_module(wanted)._numba_memory_manager)
+    except Exception:
+        raise RuntimeError("Failed to use memory manager from %s" % wanted)
 
 
 # --------------------------------------------------------------------------------
 # Context
 # --------------------------------------------------------------------------------
 
+HIP_STREAM_PER_THREAD = 2
+
+
+class _ResultCells:
+    """16-byte cells in page-locked, device-mapped host memory.  A reduction that
+    returns its value to the caller has the kernel write it into a cell and reads it
+    after waiting for the stream: no device-to-host copy, which would cost as much
+    again as the launch.  Every call takes a cell of its own and gives it back after
+    reading, so calls on any mix of host threads and streams never share one."""
+
+    CELL = 16
+    BLOCK = 4096
+
+    def __init__(self):
+        self._lock = threading.Lock()
+        self._blocks = []       # (host address, uint8 array over the block)
+        self._free = []         # (device address, uint8 view of the cell)
+
+    def take(self):
+        try:
+            return self._free.pop()
+        except IndexError:
+            pass
+        with self._lock:
+            if not self._free:
+                host, dev = c_void_p(), c_void_p()
+                driver.nbh_host_alloc(byref(host), self.BLOCK, 2)       # 2: device-mapped
+                driver.nbh_host_get_device_pointer(byref(dev), host.value)
+                raw = np.frombuffer((ctypes.c_ubyte * self.BLOCK).from_address(host.value), dtype=np.uint8)
+                self._blocks.append((host.value, raw))
+                for off in range(0, self.BLOCK, self.CELL):
+                    self._free.append((dev.value + off, raw[off:off + self.CELL]))
+            return self._free.pop()
+
+    def give_back(self, cell):
+        self._free.append(cell)
+
+    def release_all(self):
+        with self._lock:
+            blocks, self._blocks, self._free = self._blocks, [], []
+        for host, _ in blocks:
+            try:
+                driver.nbh_host_free(host)
+            except Exception:
+                pass
+
+
 class Context:
     """Per-device state (reference: Context :1061-1301)."""
 
     def __init__(self, device):
-        self.device = device
-        self.handle = device.id
-        self.deallocations = _PendingDeallocs()
-        _ensure_memory_manager()
-        self.memory_manager = _memory_manager(context=self)
+        self.device, self.handle = device, device.id
         self.extras = {}
-        self._scratch = {}   # stream handle -> device scratch for nbh_reduce
-        self._result_slots = {}   # stream handle -> host-mapped slot for results that go back to the caller
+        self.deallocations = _PendingDeallocs()      # streams and events; memory waits in the manager's queue
+        _ensure_memory_manager()
+        manager_class = _memory_manager
+        self.memory_manager = manager_class(context=self)
+        self._scratch_lock = threading.Lock()
+        self._scratch = {}          # stream handle -> (address, bytes, memory) of nbh_reduce's scratch
+        self._scratch_tls = threading.local()   # the same for each thread's per-thread default stream
+        self._result_cells = _ResultCells()
 
     @property
     def memory_manager(self):
@@ -530,48 +697,67 @@ class Context:
 
     def reset(self):
         _logger.info("reset context of device %s", self.device.id)
-        self._scratch.clear()
-        self._free_result_slots()
-        self.memory_manager.reset()
+        with self._scratch_lock:
+            self._scratch.clear()
+        self._scratch_tls = threading.local()
+        self._result_cells.release_all()
+        self._memory_manager.reset()
         self.deallocations.clear()
 
     def prepare_for_use(self):
-        self.memory_manager.initialize()
+        """Called whenever the context is fetched: lets the manager initialise (once)."""
+        self._memory_manager.initialize()
         self.prepared = True
+
+    # --- memory: all of it is the memory manager's business
+
+    def get_memory_info(self):
+        """(free, total) bytes of device memory."""
+        return self._memory_manager.get_memory_info()
+
+    def memalloc(self, bytesize):
+        """Device memory -> owned MemoryPointer."""
+        return self._memory_manager.memalloc(bytesize)
+
+    def memallocmanaged(self, bytesize, attach_global=True):
+        """Memory with one address valid on host and device."""
+        return self._memory_manager.memallocmanaged(bytesize, attach_global)
+
+    def memhostalloc(self, bytesize, mapped=False, portable=False, wc=False):
+        """Page-locked host memory, optionally addressable from the device."""
+        return self._memory_manager.memhostalloc(bytesize, mapped, portable, wc)
+
+    def mempin(self, owner, pointer, size, mapped=False):
+        """Page-lock `size` bytes of existing host memory at `pointer`."""
+        if mapped and not self.device.CAN_MAP_HOST_MEMORY:
+            raise CudaDriverError("%s cannot map host memory" % self.device)
+        return self._memory_manager.mempin(owner, pointer, size, mapped)
+
+    def defer_cleanup(self):
+        """Context manager: neither the manager's nor the context's waiting
+        releases are carried out inside."""
+        return _Both(self._memory_manager.defer_cleanup(), self.deallocations.disable())
+
+    # --- sharing memory with other processes
 
     def get_ipc_handle(self, memory):
         """An IpcHandle for `memory`, to be sent to another process (reference :1190-1198)."""
         if not sys.platform.startswith("linux"):
             raise OSError("OS does not support CUDA IPC")
-        return self.memory_manager.get_ipc_handle(memory)
+        return self._memory_manager.get_ipc_handle(memory)
 
     def open_ipc_handle(self, handle, size):
         """Map the allocation `handle` names into this process; `size` bytes of it
         will be used (reference :1200-1209).  IpcHandle.close() unmaps it."""
-        dptr = c_void_p()
-        driver.nbh_ipc_open(byref(dptr), bytes(handle.reserved), size)
-        return MemoryPointer(context=weakref.proxy(self), pointer=dptr, size=size)
+        mapped_at = c_void_p()
+        driver.nbh_ipc_open(byref(mapped_at), bytes(handle.reserved), size)
+        return MemoryPointer(context=weakref.proxy(self), pointer=mapped_at, size=size)
 
     def can_access_peer(self, peer_device):
         """One device per process here: only the device itself is reachable."""
         return int(peer_device) == self.device.id
 
-    def get_memory_info(self):
-        return self.memory_manager.get_memory_info()
-
-    def memalloc(self, bytesize):
-        return self.memory_manager.memalloc(bytesize)
-
-    def memhostalloc(self, bytesize, mapped=False, portable=False, wc=False):
-        return self.memory_manager.memhostalloc(bytesize, mapped, portable, wc)
-
-    def memallocmanaged(self, bytesize, attach_global=True):
-        return self.memory_manager.memallocmanaged(bytesize, attach_global)
-
-    def mempin(self, owner, pointer, size, mapped=False):
-        if mapped and not self.device.CAN_MAP_HOST_MEMORY:
-            raise CudaDriverError("%s cannot map host memory" % self.device)
-        return self.memory_manager.mempin(owner, pointer, size, mapped)
+    # --- streams and events
 
     def get_default_stream(self):
         return Stream(0)
@@ -583,154 +769,118 @@ class Context:
         return Stream(HIP_STREAM_PER_THREAD)
 
     def create_stream(self):
-        h = c_void_p()
-        driver.nbh_stream_create(byref(h))
-        handle = h.value or 0
-        return Stream(handle, finalizer=_stream_finalizer(self.deallocations, handle))
+        out = c_void_p()
+        driver.nbh_stream_create(byref(out))
+        handle = out.value or 0
+        return Stream(handle, finalizer=_StreamGone(self, handle))
 
     def create_external_stream(self, ptr):
-        if not isinstance(ptr, int):
-            raise TypeError("ptr for external stream must be an int")
-        return Stream(ptr, external=True)
+        if isinstance(ptr, int):
+            return Stream(ptr, external=True)
+        raise TypeError("ptr for external stream must be an int")
 
     def create_event(self, timing=True):
-        h = c_void_p()
-        driver.nbh_event_create(byref(h), 1 if timing else 0)
-        handle = h.value or 0
-        return Event(handle, finalizer=_event_finalizer(self.deallocations, handle))
+        out = c_void_p()
+        driver.nbh_event_create(byref(out), 1 if timing else 0)
+        handle = out.value or 0
+        return Event(handle, finalizer=_Release(_destroy_event, handle, queue=self.deallocations))
 
     def synchronize(self):
         driver.nbh_device_synchronize()
 
-    @contextlib.contextmanager
-    def defer_cleanup(self):
-        with self.memory_manager.defer_cleanup():
-            with self.deallocations.disable():
-                yield
-
-    _RESULT_SLOT_BYTES = 256
+    # --- what nbh_reduce needs besides its input and output
 
     def reduce_scratch(self, stream_handle):
-        """(scratch address, result slot address, scratch size) for nbh_reduce on
-        the given stream, made and zeroed on first use.  Work on one stream is
-        ordered, so consecutive reductions on it can share both; different streams
-        get their own.  The slot sits behind the scratch area in the same
-        allocation."""
+        """(address, size) of the scratch buffer (ticket + partials) for reductions
+        on the given stream, allocated and zeroed on first use.
+
+        Work on one stream runs in order, so every reduction on it can share one
+        buffer, from any host thread; different streams may overlap and get their
+        own.  The per-thread default stream is a different stream in every host
+        thread under one handle: its buffer is kept per thread and goes away with
+        the thread.  A buffer is released when its Stream object is destroyed."""
+        if stream_handle == HIP_STREAM_PER_THREAD:
+            entry = getattr(self._scratch_tls, "entry", None)
+            if entry is None:
+                entry = self._scratch_tls.entry = self._new_scratch()
+            return entry[0], entry[1]
         entry = self._scratch.get(stream_handle)
         if entry is None:
-            nbytes = driver.lib.nbh_reduce_scratch_bytes()
-            mem = self.memalloc(nbytes + self._RESULT_SLOT_BYTES)
-            ptr = mem.device_ctypes_pointer.value
-            driver.nbh_memset8(ptr, 0, nbytes + self._RESULT_SLOT_BYTES, None)
-            entry = self._scratch[stream_handle] = (ptr, ptr + nbytes, nbytes, mem)
-        return entry[0], entry[1], entry[2]
+            with self._scratch_lock:
+                entry = self._scratch.get(stream_handle)
+                if entry is None:
+                    entry = self._scratch[stream_handle] = self._new_scratch()
+        return entry[0], entry[1]
 
-    def reduce_result_slot(self, stream_handle, dtype):
-        """(device-visible address, one-item host array) of a result slot in page-locked,
-        device-mapped host memory: a reduction that returns its value to the caller
-        writes it there, and the host reads it after waiting for the stream - no
-        device-to-host copy (which costs as much again as the launch).  One slot per
-        stream, viewed through the dtype asked for."""
-        entry = self._result_slots.get(stream_handle)
-        if entry is None:
-            host = c_void_p()
-            driver.nbh_host_alloc(byref(host), self._RESULT_SLOT_BYTES, 2)       # 2: device-mapped
-            dev = c_void_p()
-            driver.nbh_host_get_device_pointer(byref(dev), host.value)
-            raw = np.frombuffer((ctypes.c_ubyte * self._RESULT_SLOT_BYTES).from_address(host.value), dtype=np.uint8)
-            entry = self._result_slots[stream_handle] = (dev.value, host.value, raw, {})
-        view = entry[3].get(dtype)
-        if view is None:
-            view = entry[3][dtype] = entry[2][:dtype.itemsize].view(dtype)
-        return entry[0], view
+    def _new_scratch(self):
+        nbytes = driver.lib.nbh_reduce_scratch_bytes()
+        mem = self.memalloc(nbytes)
+        address = mem.device_ctypes_pointer.value
+        driver.nbh_memset8(address, 0, nbytes, None)
+        return address, nbytes, mem
 
-    def _free_result_slots(self):
-        slots, self._result_slots = self._result_slots, {}
-        for _, host, _, _ in slots.values():
-            try:
-                driver.nbh_host_free(host)
-            except Exception:
-                pass
+    def _forget_stream(self, stream_handle):
+        """The stream is about to be destroyed: let go of what was kept for it."""
+        with self._scratch_lock:
+            self._scratch.pop(stream_handle, None)
+
+    def take_result_cell(self):
+        """(device address, 16 host bytes as a uint8 array) for one result; hand it
+        back with give_back_result_cell() after reading."""
+        return self._result_cells.take()
+
+    def give_back_result_cell(self, cell):
+        self._result_cells.give_back(cell)
 
     def __repr__(self):
         return "<HIP context of device %d>" % self.device.id
 
     def __eq__(self, other):
-        return isinstance(other, Context) and self.handle == other.handle
+        return isinstance(other, Context) and other.handle == self.handle
 
     def __hash__(self):
-        return hash(("ctx", self.handle))
+        return hash(("hip-context", self.handle))
 
 
-HIP_STREAM_PER_THREAD = 2
+class _Both:
+    """Two context managers entered together, left in reverse order."""
+
+    def __init__(self, outer, inner):
+        self._outer, self._inner = outer, inner
+
+    def __enter__(self):
+        self._outer.__enter__()
+        try:
+            self._inner.__enter__()
+        except BaseException:
+            self._outer.__exit__(*sys.exc_info())
+            raise
+
+    def __exit__(self, *exc):
+        try:
+            self._inner.__exit__(*exc)
+        finally:
+            self._outer.__exit__(*exc)
+        return False
 
 
-def _alloc_finalizer(memory_manager, ptr, alloc_key, size):
-    allocations = memory_manager.allocations
-    deallocations = memory_manager.deallocations
+class _StreamGone:
+    """Finalizer of a created stream: the context drops the scratch it kept for the
+    stream (queued kernels may still use it - its free waits in the queue, and
+    hipFree waits for the device), then the destroy call is parked too."""
 
-    def core():
-        if allocations:
-            allocations.pop(alloc_key, None)
-        deallocations.add_item(_free_device, ptr, size)
+    __slots__ = ("context", "handle")
 
-    return core
+    def __init__(self, context, handle):
+        self.context = weakref.ref(context)
+        self.handle = handle
 
-
-def _hostalloc_finalizer(memory_manager, ptr, alloc_key, size, mapped):
-    allocations = memory_manager.allocations
-    deallocations = memory_manager.deallocations
-    if not mapped:
-        size = _SizeNotSet
-
-    def core():
-        if mapped and allocations:
-            allocations.pop(alloc_key, None)
-        deallocations.add_item(_free_host, ptr, size)
-
-    return core
-
-
-def _pin_finalizer(memory_manager, ptr, alloc_key, mapped):
-    # unregistering cannot wait: the same host buffer may be pinned again at once
-    allocations = memory_manager.allocations
-
-    def core():
-        if mapped and allocations:
-            allocations.pop(alloc_key, None)
-        driver.nbh_host_unregister(ptr)
-
-    return core
-
-
-def _free_device(ptr):
-    driver.nbh_free(ptr)
-
-
-def _free_host(ptr):
-    driver.nbh_host_free(ptr)
-
-
-def _destroy_stream(handle):
-    driver.nbh_stream_destroy(handle)
-
-
-def _destroy_event(handle):
-    driver.nbh_event_destroy(handle)
-
-
-def _event_finalizer(deallocs, handle):
-    def core():
-        deallocs.add_item(_destroy_event, handle)
-
-    return core
-
-
-def _stream_finalizer(deallocs, handle):
-    def core():
-        deallocs.add_item(_destroy_stream, handle)
-
-    return core
+    def __call__(self):
+        ctx = self.context()
+        if ctx is None:
+            return
+        ctx._forget_stream(self.handle)
+        ctx.deallocations.add_item(_destroy_stream, self.handle)
 
 
 # --------------------------------------------------------------------------------
@@ -758,32 +908,6 @@ class IpcMemHandle:
         self._reserved = value
 
 
-class _DirectIpc:
-    """An imported mapping of the exporter's allocation."""
-
-    def __init__(self, parent):
-        self.parent = parent
-        self._opened = None
-
-    def open(self, context):
-        p = self.parent
-        if p.base is not None:
-            raise ValueError("opening IpcHandle from original process")
-        if self._opened is not None:
-            raise ValueError("IpcHandle is already opened")
-        if p.offset + p.size >= IPC_ALLOCATION_LIMIT:
-            raise ValueError("allocations of 2 GiB or more cannot be shared between processes")
-        mem = context.open_ipc_handle(p.handle, p.offset + p.size)
-        self._opened = mem            # this object owns the mapping until close()
-        return mem.own().view(p.offset)
-
-    def close(self):
-        if self._opened is None:
-            raise ValueError("IpcHandle not opened")
-        driver.nbh_ipc_close(self._opened.handle)
-        self._opened = None
-
-
 class IpcHandle:
     """A picklable name for a device allocation that another process on the same
     machine can open (reference :1487-1603).
@@ -793,63 +917,63 @@ class IpcHandle:
     size        bytes of the shared region
     source_info identity of the exporting device
     offset      where the region starts in the underlying allocation
-    """
+
+    In the importing process open() maps the exporter's allocation and close()
+    unmaps it; the handle owns the mapping in between."""
 
     def __init__(self, base, handle, size, source_info=None, offset=0):
-        self.base = base
-        self.handle = handle
-        self.size = size
-        self.source_info = source_info
-        self.offset = offset
-        self._impl = None
+        self.base, self.handle, self.size = base, handle, size
+        self.source_info, self.offset = source_info, offset
+        self._mapping = None        # MemoryPointer over the imported allocation while open
 
-    def _sentry_source_info(self):
+    def _refuse_if_open(self):
+        if self._mapping is not None:
+            raise ValueError("IpcHandle is already opened")
+
+    def _need_source_info(self):
         if self.source_info is None:
             raise RuntimeError("IPC handle doesn't have source info")
 
     def can_access_peer(self, context):
-        self._sentry_source_info()
-        if self.source_info == context.device.get_device_identity():
-            return True
-        return context.can_access_peer(Device.from_identity(self.source_info).id)
+        self._need_source_info()
+        here = context.device.get_device_identity()
+        return self.source_info == here or context.can_access_peer(Device.from_identity(self.source_info).id)
 
     def open_staged(self, context):
         """Copy through the exporting device when the importer cannot reach it.  That
         needs a second device in the importing process, which this build never has."""
-        self._sentry_source_info()
-        if self._impl is not None:
-            raise ValueError("IpcHandle is already opened")
+        self._need_source_info()
+        self._refuse_if_open()
         raise NotImplementedError("staged IPC between two devices is not part of this build")
 
     def open_direct(self, context):
-        if self._impl is not None:
-            raise ValueError("IpcHandle is already opened")
-        self._impl = _DirectIpc(self)
-        try:
-            return self._impl.open(context)
-        except Exception:
-            self._impl = None
-            raise
+        self._refuse_if_open()
+        if self.base is not None:
+            raise ValueError("opening IpcHandle from original process")
+        wanted = self.offset + self.size
+        if wanted >= IPC_ALLOCATION_LIMIT:
+            raise ValueError("allocations of 2 GiB or more cannot be shared between processes")
+        self._mapping = context.open_ipc_handle(self.handle, wanted)
+        return self._mapping.own().view(self.offset)
 
     def open(self, context):
         """Map the memory into `context`'s process -> device memory pointer."""
-        if self.source_info is None or self.can_access_peer(context):
-            return self.open_direct(context)
-        return self.open_staged(context)
+        if self.source_info is not None and not self.can_access_peer(context):
+            return self.open_staged(context)
+        return self.open_direct(context)
 
     def open_array(self, context, shape, dtype, strides=None):
         """open(), wrapped as a device array (1-d C-contiguous unless `strides` says otherwise)."""
         from numba_cuda_amd.cudadrv import devicearray
-        if strides is None:
-            strides = dtype.itemsize
-        dptr = self.open(context)
-        return devicearray.DeviceNDArray(shape=shape, strides=strides, dtype=dtype, gpu_data=dptr)
+        memory = self.open(context)
+        return devicearray.DeviceNDArray(shape=shape, strides=dtype.itemsize if strides is None else strides,
+                                         dtype=dtype, gpu_data=memory)
 
     def close(self):
-        if self._impl is None:
+        if self._mapping is None:
             raise ValueError("IpcHandle not opened")
-        self._impl.close()
-        self._impl = None
+        mapping, self._mapping = self._mapping, None
+        driver.nbh_ipc_close(mapping.handle)
 
     def __reduce__(self):
         return (_rebuild_ipc_handle, (self.__class__, self.handle.reserved, self.size, self.source_info, self.offset))
@@ -864,73 +988,92 @@ def _rebuild_ipc_handle(cls, *args):
 
 
 class MemoryPointer:
-    """A device buffer (reference :1606-1717).  `refct` counts the owned
-    references handed out by own()/view(); for the base class the buffer lives as
-    long as the instance, for AutoFreePointer as long as refct > 0."""
+    """A range of device memory (reference :1606-1717).
+
+    `refct` counts the references handed out by own() and view(), plus one for the
+    object itself: a plain MemoryPointer therefore never drops to zero and its
+    buffer lives exactly as long as the object (the finalizer, when one was given,
+    runs when the object is collected or free() is called).  AutoFreePointer leaves
+    the one for itself out, so there the last owned reference ends the buffer.
+
+    `owner` is the object the buffer belongs to: the pointer itself, the pointer a
+    view was cut from, or whatever foreign object was passed as `owner`."""
 
     __cuda_memory__ = True
+    _counts_itself = 1
 
     def __init__(self, context, pointer, size, owner=None, finalizer=None):
         if isinstance(pointer, (c_void_p, c_size_t)):
             pointer = pointer.value
-        address = int(pointer or 0)
-        self.context, self._owner = context, owner
-        self.device_pointer = self.handle = address
+        self.context = context
+        self.handle = self.device_pointer = int(pointer or 0)
         self.size = self._cuda_memsize_ = size
-        self.refct = 1
+        self._owner = owner
+        self.refct = self._counts_itself
         self.is_managed = finalizer is not None
-        if self.is_managed:
-            self._finalizer = weakref.finalize(self, finalizer)
+        self._finalizer = weakref.finalize(self, finalizer) if self.is_managed else None
 
     @property
     def owner(self):
-        return self if self._owner is None else self._owner
+        return self._owner if self._owner is not None else self
 
-    def own(self):
-        return OwnedPointer(weakref.proxy(self))
-
-    def free(self):
-        """Send the buffer to the pending-deallocation queue now."""
-        if self.is_managed:
-            if not self._finalizer.alive:
-                raise RuntimeError("Freeing dead memory")
-            self._finalizer()
-            assert not self._finalizer.alive
-
-    def memset(self, byte, count=None, stream=0):
-        count = self.size if count is None else count
-        driver.nbh_memset8(self.device_pointer, byte, count, _stream_handle(stream) or None)
-
-    def view(self, start, stop=None):
-        size = (self.size - start) if stop is None else (stop - start)
-        if not self.device_pointer_value:
-            if size != 0:
-                raise RuntimeError("non-empty slice into empty slice")
-            view = self
-        else:
-            if size < 0:
-                raise RuntimeError("size cannot be negative")
-            view = MemoryPointer(self.context, self.device_pointer_value + start, size, owner=self.owner)
-        if isinstance(self.owner, (MemoryPointer, OwnedPointer)):
-            # the owner is memory we manage: the view holds a counted reference
-            return OwnedPointer(weakref.proxy(self.owner), view)
-        return view   # foreign owner: the view just carries it along
+    @property
+    def device_pointer_value(self):
+        """The address, or None for a null pointer."""
+        return self.device_pointer or None
 
     @property
     def device_ctypes_pointer(self):
         return c_size_t(self.device_pointer)
 
-    @property
-    def device_pointer_value(self):
-        return self.device_pointer or None
+    def own(self):
+        """A counted reference to this memory."""
+        return OwnedPointer(weakref.proxy(self))
+
+    def _let_go(self):
+        """One counted reference less; the last one ends the buffer."""
+        self.refct -= 1
+        if self.refct == 0:
+            self.free()
+        elif self.refct < 0:
+            raise AssertionError("memory reference count below zero")
+
+    def free(self):
+        """Run the finalizer now (the raw free then waits in the queue)."""
+        hook = self._finalizer
+        if hook is None:
+            return
+        if not hook.alive:
+            raise RuntimeError("Freeing dead memory")
+        hook()
+
+    def memset(self, byte, count=None, stream=0):
+        nbytes = self.size if count is None else count
+        driver.nbh_memset8(self.device_pointer, byte, nbytes, _stream_handle(stream) or None)
+
+    def view(self, start, stop=None):
+        """Pointer to bytes [start, stop) of this one (to the end without `stop`).
+        When the buffer is memory managed here, the result holds a counted reference
+        to the owner; with a foreign owner it simply carries that owner along."""
+        nbytes = (self.size if stop is None else stop) - start
+        if self.device_pointer_value is None:
+            if nbytes:
+                raise RuntimeError("non-empty slice into empty slice")
+            piece = self                     # a view of nothing is the nothing itself
+        elif nbytes < 0:
+            raise RuntimeError("size cannot be negative")
+        else:
+            piece = MemoryPointer(self.context, self.device_pointer + start, nbytes, owner=self.owner)
+        root = self.owner
+        if isinstance(root, (MemoryPointer, OwnedPointer)):
+            return OwnedPointer(weakref.proxy(root), piece)
+        return piece
 
 
 class AutoFreePointer(MemoryPointer):
-    """Freed when the last owned reference goes away (reference :1719-1733)."""
+    """Device memory that ends with its last owned reference (reference :1719-1733)."""
 
-    def __init__(self, *args, **kwargs):
-        super().__init__(*args, **kwargs)
-        self.refct -= 1
+    _counts_itself = 0
 
 
 class _HostBufferMixin(_hostbuf.HostBuffer):
@@ -942,21 +1085,24 @@ class _HostBufferMixin(_hostbuf.HostBuffer):
     def as_buffer(self):
         return self
 
+    def _export(self, address, nbytes):
+        self.host_pointer = self._bufptr_ = address
+        self._buflen_ = nbytes
+
 
 class MappedMemory(AutoFreePointer, _HostBufferMixin):
-    """Page-locked host memory that is also addressable from the device."""
-
-    __cuda_memory__ = True
+    """Page-locked host memory that is also addressable from the device
+    (reference :1735-1768).  `handle` is the host address, `device_pointer` the
+    address kernels use."""
 
     def __init__(self, context, pointer, size, owner=None, finalizer=None):
+        host_address = int(pointer)
+        seen_from_device = c_void_p()
+        driver.nbh_host_get_device_pointer(byref(seen_from_device), host_address)
+        super().__init__(context, seen_from_device.value or 0, size, finalizer=finalizer)
         self.owned = owner
-        self.host_pointer = int(pointer)
-        devptr = c_void_p()
-        driver.nbh_host_get_device_pointer(byref(devptr), self.host_pointer)
-        super().__init__(context, devptr.value or 0, size, finalizer=finalizer)
-        self.handle = self.host_pointer
-        self._bufptr_ = self.host_pointer
-        self._buflen_ = self.size
+        self.handle = host_address
+        self._export(host_address, size)
 
     def own(self):
         return MappedOwnedPointer(weakref.proxy(self))
@@ -966,72 +1112,62 @@ class ManagedMemory(AutoFreePointer, _HostBufferMixin):
     """Managed memory: one address, valid on the host and on the device
     (reference :1813-1845)."""
 
-    __cuda_memory__ = True
-
     def __init__(self, context, pointer, size, owner=None, finalizer=None):
-        self.owned = owner
         super().__init__(context, int(pointer), size, finalizer=finalizer)
-        self.host_pointer = int(pointer)
-        self._bufptr_ = self.host_pointer
-        self._buflen_ = self.size
+        self.owned = owner
+        self._export(self.device_pointer, size)
 
     def own(self):
         return ManagedOwnedPointer(weakref.proxy(self))
 
 
 class PinnedMemory(_HostBufferMixin):
-    """Page-locked host memory (reference :1770-1808)."""
+    """Page-locked host memory the device cannot address (reference :1770-1808).
+    Not reference counted: own() is the object itself, and the finalizer runs when
+    it is collected."""
 
     def __init__(self, context, pointer, size, owner=None, finalizer=None):
-        self.context = context
-        self.owned = owner
-        self.size = size
-        self.host_pointer = int(pointer)
-        self.is_managed = finalizer is not None
+        self.context, self.owned, self.size = context, owner, size
+        self._export(int(pointer), size)
         self.handle = self.host_pointer
-        self._buflen_ = self.size
-        self._bufptr_ = self.host_pointer
-        if finalizer is not None:
-            weakref.finalize(self, finalizer)
+        self.is_managed = bool(finalizer is not None)
+        self._finalizer = weakref.finalize(self, finalizer) if self.is_managed else None
 
     def own(self):
         return self
 
 
+def _let_go(memory):
+    try:
+        memory._let_go()
+    except ReferenceError:
+        pass      # the memory object went first; nothing left to release
+
+
 class OwnedPointer:
     """A counted reference to a MemoryPointer, optionally looking at a sub-range
     of it (reference :1848-1880).  Creating one bumps the owner's `refct`; when it
-    is collected the count drops again and the owner is freed at zero.  Attribute
-    access falls through to the pointer it looks at."""
+    is collected the count drops again.  Every attribute not found here is the
+    attribute of the pointer it looks at."""
 
     def __init__(self, memptr, view=None):
-        target = memptr if view is None else view
-        if view is not None:
-            assert not view.is_managed
-        self._mem, self._view = memptr, target
-        # used on every kernel argument: worth a real attribute
-        self.device_ctypes_pointer = target.device_ctypes_pointer
+        if view is not None and view.is_managed:
+            raise AssertionError("a view into owned memory cannot have a finalizer of its own")
+        self._mem = memptr
+        self._view = memptr if view is None else view
+        # read for every kernel argument: worth a real attribute
+        self.device_ctypes_pointer = self._view.device_ctypes_pointer
         memptr.refct += 1
-        weakref.finalize(self, _drop_reference, memptr)
+        weakref.finalize(self, _let_go, memptr)
 
-    def __getattr__(self, fname):
-        return getattr(self._view, fname)
+    def __getattr__(self, name):
+        return getattr(self._view, name)
 
     def view(self, start, stop=None):
         # a real method rather than a fall-through: in `ctx.memalloc(n).view(k)` the
         # temporary reference must outlive the call, or the memory is freed before the
         # derived pointer has taken its own reference
         return self._view.view(start, stop)
-
-
-def _drop_reference(mem):
-    try:
-        mem.refct -= 1
-        assert mem.refct >= 0
-        if mem.refct == 0:
-            mem.free()
-    except ReferenceError:
-        pass      # the owner went first; nothing left to release
 
 
 class MappedOwnedPointer(OwnedPointer, _HostBufferMixin):
@@ -1045,6 +1181,24 @@ class ManagedOwnedPointer(OwnedPointer, _HostBufferMixin):
 # --------------------------------------------------------------------------------
 # Streams and events
 # --------------------------------------------------------------------------------
+
+class _SyncOnExit:
+    """`with stream.auto_synchronize():` - wait for the stream when the block is
+    left normally."""
+
+    __slots__ = ("_stream",)
+
+    def __init__(self, stream):
+        self._stream = stream
+
+    def __enter__(self):
+        return self._stream
+
+    def __exit__(self, exc_type, exc, tb):
+        if exc_type is None:
+            self._stream.synchronize()
+        return False
+
 
 class Stream:
     """A HIP stream; handle 0 is the legacy default stream (reference :1890-2017)."""
@@ -1086,17 +1240,16 @@ class Stream:
     def query(self):
         return _query(driver.lib.nbh_stream_query(self.handle or None), "nbh_stream_query")
 
-    @contextlib.contextmanager
     def auto_synchronize(self):
-        yield self
-        self.synchronize()
+        return _SyncOnExit(self)
 
     def add_callback(self, callback, arg=None):
         """Call `callback(stream, status, arg)` from a runtime thread once everything
         queued on this stream so far has finished (status is 0).  The callback must
         not call back into the GPU API and should be short: later work on the stream
         waits for it."""
-        token = object()
+        _drain_finished_thunks()
+        slot = []
 
         def trampoline(_user):
             try:
@@ -1105,14 +1258,17 @@ class Stream:
                 import warnings
                 warnings.warn("Exception in stream callback: %s" % (e,))
             finally:
-                _live_callbacks.pop(token, None)
+                # The native thunk is still executing: it must not lose its last
+                # reference here.  It moves to a list that later calls empty.
+                _finished_thunks.append(_pending_thunks.pop(id(slot), None))
 
-        cfn = _lib.HOST_FN(trampoline)
-        _live_callbacks[token] = cfn          # keep the thunk alive until it has run
+        thunk = _lib.HOST_FN(trampoline)
+        slot.append(thunk)
+        _pending_thunks[id(slot)] = (thunk, slot)
         try:
-            driver.nbh_stream_add_callback(self.handle or None, cfn, None)
+            driver.nbh_stream_add_callback(self.handle or None, thunk, None)
         except Exception:
-            _live_callbacks.pop(token, None)
+            _pending_thunks.pop(id(slot), None)
             raise
 
     def async_done(self):
@@ -1121,22 +1277,28 @@ class Stream:
         loop = asyncio.get_running_loop()
         future = loop.create_future()
 
-        def resolver(fut, status):
-            if fut.done():
+        def settle(status):
+            if future.done():
                 return
             if status == 0:
-                fut.set_result(self)
+                future.set_result(self)
             else:
-                fut.set_exception(Exception("Stream error %s" % status))
+                future.set_exception(Exception("Stream error %s" % status))
 
-        def callback(stream, status, fut):
-            loop.call_soon_threadsafe(resolver, fut, status)
-
-        self.add_callback(callback, future)
+        self.add_callback(lambda _stream, status, _arg: loop.call_soon_threadsafe(settle, status))
         return future
 
 
-_live_callbacks = {}
+_pending_thunks = {}     # id -> (thunk, holder) of callbacks that have not run yet
+_finished_thunks = []    # thunks whose callback has run; dropped by a later call
+
+
+def _drain_finished_thunks():
+    # everything that was in the list when we got here returned from its thunk
+    # at least one Python-level call ago
+    n = len(_finished_thunks)
+    if n > 64:
+        del _finished_thunks[:n - 8]
 
 
 def _query(code, fname):
@@ -1154,20 +1316,22 @@ class Event:
         if finalizer is not None:
             weakref.finalize(self, finalizer)
 
+    def record(self, stream=0):
+        driver.nbh_event_record(self.handle, _stream_handle(stream) or None)
+
+    def wait(self, stream=0):
+        """Work queued on `stream` after this call starts after the event."""
+        driver.nbh_stream_wait_event(_stream_handle(stream) or None, self.handle)
+
     def query(self):
         driver.ensure_initialized()
         return _query(driver.lib.nbh_event_query(self.handle), "nbh_event_query")
 
-    def record(self, stream=0):
-        driver.nbh_event_record(self.handle, _stream_handle(stream) or None)
-
     def synchronize(self):
         driver.nbh_event_synchronize(self.handle)
 
-    def wait(self, stream=0):
-        driver.nbh_stream_wait_event(_stream_handle(stream) or None, self.handle)
-
     def elapsed_time(self, evtend):
+        """Milliseconds from this event to `evtend`."""
         return event_elapsed_time(self, evtend)
 
 
@@ -1179,30 +1343,31 @@ def event_elapsed_time(evtstart, evtend):
 
 
 def _stream_handle(stream):
-    """0 or a Stream object -> raw handle (reference :2767-2789)."""
+    """0 or a Stream object (or anything with __cuda_stream__) -> raw handle
+    (reference :2767-2789)."""
     if isinstance(stream, Stream):
         return stream.handle
     if isinstance(stream, int) and stream == 0:
         return 0
-    if hasattr(stream, "__cuda_stream__"):
-        ver, ptr = stream.__cuda_stream__()
-        assert ver == 0
-        return int(ptr)
-    raise TypeError("Expected a Stream object or 0, got %s" % type(stream).__name__)
+    protocol = getattr(stream, "__cuda_stream__", None)
+    if protocol is None:
+        raise TypeError("Expected a Stream object or 0, got %s" % type(stream).__name__)
+    version, address = protocol()
+    if version != 0:
+        raise TypeError("__cuda_stream__ protocol version %r is not supported" % (version,))
+    return int(address)
 
 
 # --------------------------------------------------------------------------------
 # Pointers, extents, copies
 # --------------------------------------------------------------------------------
 
-def _is_datetime_dtype(obj):
+def _plain_view(obj):
+    # datetime64 / timedelta64 arrays do not export a buffer; their int64 view does
     dtype = getattr(obj, "dtype", None)
-    return dtype is not None and dtype.char in "Mm"
-
-
-def _workaround_for_datetime(obj):
-    # datetime64 / timedelta64 do not export a buffer; their int64 view does
-    return obj.view(np.int64) if _is_datetime_dtype(obj) else obj
+    if dtype is not None and dtype.char in "Mm":
+        return obj.view(np.int64)
+    return obj
 
 
 def host_pointer(obj, readonly=False):
@@ -1210,7 +1375,7 @@ def host_pointer(obj, readonly=False):
     Accepts an int, a NumPy array or scalar, or any buffer-protocol object."""
     if isinstance(obj, int):
         return obj
-    obj = _workaround_for_datetime(obj)
+    obj = _plain_view(obj)
     if isinstance(obj, np.ndarray):
         if not readonly and not obj.flags.writeable:
             raise BufferError("writable buffer requested from a read-only array")
@@ -1229,7 +1394,8 @@ def _extents(ptr, shape, strides, itemsize):
 
 
 def host_memory_extents(obj):
-    obj = _workaround_for_datetime(obj)
+    """[begin, end) addresses a host object's data occupies."""
+    obj = _plain_view(obj)
     if isinstance(obj, (np.ndarray, np.generic)):
         a = np.asarray(obj)
         return _extents(a.__array_interface__["data"][0], a.shape, a.strides, a.itemsize)
@@ -1237,64 +1403,84 @@ def host_memory_extents(obj):
 
 
 def host_memory_size(obj):
-    s, e = host_memory_extents(obj)
-    assert e >= s, "memory extend of negative size"
-    return e - s
+    begin, end = host_memory_extents(obj)
+    if end < begin:
+        raise AssertionError("memory extent of negative size")
+    return end - begin
 
 
-@functools.lru_cache(maxsize=4096)
+_SIZE_FROM_INFO = {}
+
+
 def memory_size_from_info(shape, strides, itemsize):
     """Bytes spanned by an array with this shape and strides, gaps included."""
-    assert len(shape) == len(strides), "# dim mismatch"
-    s, e = _extents(0, shape, strides, itemsize)
-    return e - s
-
-
-def device_pointer(obj):
-    return device_ctypes_pointer(obj).value
-
-
-def device_ctypes_pointer(obj):
-    if obj is None:
-        return c_void_p(0)
-    require_device_memory(obj)
-    return obj.device_ctypes_pointer
+    key = (shape, strides, itemsize)
+    try:
+        return _SIZE_FROM_INFO[key]
+    except KeyError:
+        pass
+    if len(shape) != len(strides):
+        raise AssertionError("# dim mismatch")
+    lo, hi = _extents(0, shape, strides, itemsize)
+    if len(_SIZE_FROM_INFO) > 4096:
+        _SIZE_FROM_INFO.clear()
+    _SIZE_FROM_INFO[key] = hi - lo
+    return hi - lo
 
 
 def is_device_memory(obj):
     """Device memory is anything with a truthy __cuda_memory__ attribute."""
-    try:
-        return obj.__cuda_memory__
-    except AttributeError:
-        return False
+    return getattr(obj, "__cuda_memory__", False)
 
 
 def require_device_memory(obj):
-    if not is_device_memory(obj):
-        raise Exception("Not a CUDA memory object.")
+    """Raise unless `obj` is device memory."""
+    if is_device_memory(obj):
+        return
+    raise Exception("Not a CUDA memory object.")
+
+
+def device_ctypes_pointer(obj):
+    """ctypes pointer of a device memory object (a null c_void_p for None)."""
+    if obj is not None:
+        require_device_memory(obj)
+        return obj.device_ctypes_pointer
+    return c_void_p(0)
+
+
+def device_pointer(obj):
+    """Address of a device memory object as an int."""
+    return device_ctypes_pointer(obj).value
 
 
 def device_extents(devmem):
     """[begin, end) of the whole allocation that `devmem` points into."""
     base, size = c_void_p(), c_size_t()
     driver.nbh_mem_address_range(byref(base), byref(size), device_ctypes_pointer(devmem).value)
-    b = base.value or 0
-    return b, b + size.value
+    begin = base.value or 0
+    return begin, begin + size.value
 
 
 def device_memory_size(devmem):
-    sz = getattr(devmem, "_cuda_memsize_", None)
-    if sz is None:
-        s, e = device_extents(devmem)
-        sz = e - s
-        devmem._cuda_memsize_ = sz
-    assert sz >= 0, "{} length array".format(sz)
-    return sz
+    """Size of the allocation behind `devmem`; looked up once and kept on the object."""
+    try:
+        known = devmem._cuda_memsize_
+    except AttributeError:
+        known = None
+    if known is None:
+        begin, end = device_extents(devmem)
+        known = devmem._cuda_memsize_ = end - begin
+    if known < 0:
+        raise AssertionError("%d length array" % known)
+    return known
 
 
 def device_memory_depends(devmem, *objs):
-    depset = getattr(devmem, "_depends_", [])
-    depset.extend(objs)
+    """Keep `objs` alive as long as `devmem` lives."""
+    kept = getattr(devmem, "_depends_", None)
+    if kept is None:
+        kept = devmem._depends_ = []
+    kept.extend(objs)
 
 
 def host_to_device(dst, src, size, stream=0):
@@ -1321,14 +1507,18 @@ def profile_start():
 
 
 def profile_stop():
-    pass
+    """See profile_start()."""
 
 
-@contextlib.contextmanager
-def profiling():
-    profile_start()
-    yield
-    profile_stop()
+class profiling:
+    """`with profiling():` - kept for source compatibility; see profile_start()."""
+
+    def __enter__(self):
+        profile_start()
+
+    def __exit__(self, *exc):
+        profile_stop()
+        return False
 
 
 def get_version():

@@ -230,48 +230,55 @@ class Reduce:
             arr, _ = devicearray.auto_device(arr, stream=stream)
 
         hstream = stream.handle if type(stream) is _driver.Stream else _driver._stream_handle(stream)
-        scratch_ptr, _, scratch_bytes = ctx.reduce_scratch(hstream)
+        scratch_ptr, scratch_bytes = ctx.reduce_scratch(hstream)
+        init_ptr = _init_buffer(dtype, init)
+        drv = _driver.driver
         if res is not None:
             if res.dtype != dtype:
                 raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
-            out_ptr = res.device_ctypes_pointer.value
-        else:
-            # per-stream slot in host memory the device can write: no allocation, no copy back
-            out_ptr, host_view = ctx.reduce_result_slot(hstream, dtype)
-        init_ptr = _init_buffer(dtype, init)
-        drv = _driver.driver
-        rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size,
-                                arr.strides[0], init_ptr,
-                                out_ptr, scratch_ptr, scratch_bytes, hstream or None)
-        if rc:
-            drv.check("nbh_reduce", rc)
-        if res is not None:
+            rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size,
+                                    arr.strides[0], init_ptr, res.device_ctypes_pointer.value,
+                                    scratch_ptr, scratch_bytes, hstream or None)
+            if rc:
+                drv.check("nbh_reduce", rc)
             return None
-        # the value is wanted on the host now: wait for the stream, then read the slot
-        drv.nbh_stream_synchronize(hstream or None)
-        return host_view[0]
+        # The value is wanted on the host: the kernel writes it into a cell of host
+        # memory the device can address (taken for this call alone, so that calls from
+        # other threads or on other streams cannot land in it), the host waits for the
+        # stream and reads the cell - no copy back.
+        cell = ctx.take_result_cell()
+        try:
+            rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size,
+                                    arr.strides[0], init_ptr, cell[0],
+                                    scratch_ptr, scratch_bytes, hstream or None)
+            if rc:
+                drv.check("nbh_reduce", rc)
+            drv.nbh_stream_synchronize(hstream or None)
+            return cell[1][:dtype.itemsize].view(dtype)[0]
+        finally:
+            ctx.give_back_result_cell(cell)
 
 
 _DTYPE_CODE = {np.dtype(name): code for name, code in _lib.DTYPE_CODES.items()}
 _BOOL = np.dtype(np.bool_)
 
 # host copies of `init` values, one element each, kept alive for the process:
-# (dtype, init) -> (array, address).  nbh_reduce reads the value during the call.
+# (dtype, bytes of the value) -> (array, address).  nbh_reduce reads the value during the call.
 _INIT_CACHE = {}
 
 
 def _init_buffer(dtype, init):
-    try:
-        return _INIT_CACHE[dtype, init][1]
-    except (KeyError, TypeError):
-        pass
+    """Address of a host copy of `init` converted to `dtype`.  The copies are kept for
+    the life of the process, found again by the bit pattern of the converted value
+    (so that 0.0 and -0.0, which compare equal, stay apart)."""
     buf = np.array([dtype.type(init)], dtype=dtype)
-    try:
-        if len(_INIT_CACHE) < 4096 and init == init:     # NaN never compares equal: do not cache it
-            _INIT_CACHE[dtype, init] = (buf, buf.ctypes.data)
-            return buf.ctypes.data
-    except TypeError:
-        pass
+    key = (dtype, buf.tobytes())
+    kept = _INIT_CACHE.get(key)
+    if kept is not None:
+        return kept[1]
+    if len(_INIT_CACHE) < 4096:
+        _INIT_CACHE[key] = (buf, buf.ctypes.data)
+        return buf.ctypes.data
     _KEEPALIVE.append(buf)
     if len(_KEEPALIVE) > 64:
         del _KEEPALIVE[:32]

@@ -26,40 +26,28 @@ from ctypes import byref, c_size_t, c_void_p
 from numba_cuda_amd.cudadrv import driver as _drv
 
 
-class PoolMemoryManager(_drv.GetIpcHandleMixin, _drv.HostOnlyCUDAMemoryManager):
-    """Device allocations from the library's caching pool; host allocations as in the
-    default manager."""
+def _back_to_pool(ptr):
+    _drv.driver.nbh_pool_free(ptr)
 
-    def initialize(self):
-        if self.deallocations.memory_capacity == _drv._SizeNotSet:
-            self.deallocations.memory_capacity = self.get_memory_info().total
+
+class PoolMemoryManager(_drv.NumbaCUDAMemoryManager):
+    """Device allocations from the library's caching pool; everything else (host
+    allocations, memory info, IPC handles) as in the default manager.
+    `get_memory_info()` reports what the driver sees: blocks idling in the pool count
+    as used (see `stats()`)."""
 
     def memalloc(self, size):
-        def allocator():
-            p = c_void_p()
-            _drv.driver.nbh_pool_malloc(byref(p), size)
-            return p.value or 0
+        def from_pool():
+            out = c_void_p()
+            _drv.driver.nbh_pool_malloc(byref(out), size)
+            return out.value or 0
 
-        ptr = self._attempt_allocation(allocator)
-        allocations = self.allocations
-
-        def finalizer():
-            # straight back to the pool: releasing a block neither frees memory nor
-            # waits for the device, so there is nothing to defer
-            if allocations:
-                allocations.pop(ptr, None)
-            _drv.driver.nbh_pool_free(ptr)
-
-        mem = _drv.AutoFreePointer(weakref.proxy(self.context), ptr, size, finalizer=finalizer)
-        self.allocations[ptr] = mem
-        return mem.own()
-
-    def get_memory_info(self):
-        """(free, total) as the driver sees them; blocks idling in the pool count as
-        used (see `stats()`)."""
-        free, total = c_size_t(), c_size_t()
-        _drv.driver.nbh_mem_info(byref(free), byref(total))
-        return _drv.MemoryInfo(free=free.value, total=total.value)
+        address = self._attempt_allocation(from_pool)
+        # straight back to the pool, not through the queue of waiting releases: giving a
+        # block back neither frees memory nor waits for the device
+        on_release = _drv._Release(_back_to_pool, address, table=self.allocations, key=address)
+        mem = _drv.AutoFreePointer(weakref.proxy(self.context), address, size, finalizer=on_release)
+        return self._track(mem, address)
 
     def reset(self):
         super().reset()
@@ -75,10 +63,6 @@ class PoolMemoryManager(_drv.GetIpcHandleMixin, _drv.HostOnlyCUDAMemoryManager):
         hits, misses = ctypes.c_uint64(), ctypes.c_uint64()
         _drv.driver.nbh_pool_stats(byref(idle), byref(live), byref(hits), byref(misses))
         return {"idle_bytes": idle.value, "live_bytes": live.value, "hits": hits.value, "misses": misses.value}
-
-    @property
-    def interface_version(self):
-        return 1
 
 
 # the hook NUMBA_CUDA_MEMORY_MANAGER=<module> looks for (reference :2751-2764)

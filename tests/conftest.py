@@ -49,7 +49,7 @@ def fake_gpu(monkeypatch):
     for name in [k for k in d.__dict__ if k.startswith("nbh_")]:
         del d.__dict__[name]                      # drop cached checked wrappers
     d.lib, d.is_initialized, d.initialization_error, d.pid = lib, True, None, os.getpid()
-    d.get_device.cache_clear()
+    d._devices = {}                               # a table of its own for the fake devices
     devices._runtime._tls.__dict__.clear()
     if "lst" in devices.gpus.__dict__:
         del devices.gpus.__dict__["lst"]
@@ -63,7 +63,6 @@ def fake_gpu(monkeypatch):
         d.__dict__.update(saved)
         for name in [k for k in d.__dict__ if k.startswith("nbh_")]:
             del d.__dict__[name]
-        d.get_device.cache_clear()
         devices._runtime._tls.__dict__.clear()
         if "lst" in devices.gpus.__dict__:
             del devices.gpus.__dict__["lst"]

@@ -28,11 +28,11 @@ def pending_byte_threshold(cuda):
     old = config.CUDA_DEALLOCS_RATIO
     try:
         config.CUDA_DEALLOCS_RATIO = max_pending / total
-        assert abs(deallocs._max_pending_bytes - max_pending) <= 1
+        assert abs(deallocs.byte_budget - max_pending) <= 1
         cuda.to_device(np.ones(max_pending // 2, dtype=np.int8))
         gc.collect()
         assert len(deallocs) == 1
-        cuda.to_device(np.ones(deallocs._max_pending_bytes - deallocs._size, dtype=np.int8))
+        cuda.to_device(np.ones(deallocs.byte_budget - deallocs.pending_bytes, dtype=np.int8))
         gc.collect()
         assert len(deallocs) == 2
         cuda.to_device(np.ones(1, dtype=np.int8))

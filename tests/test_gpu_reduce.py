@@ -336,3 +336,56 @@ def test_strided_and_reversed_views():
     assert abs(float(sum_reduce(col)) - exact) <= 2 * 300 * np.finfo(np.float32).eps * sum_abs
     b = rng.integers(-128, 127, 70_001).astype(np.int8)
     assert sum_reduce(cuda.to_device(b)[::3]) == cref.fold("add", np.ascontiguousarray(b[::3]))
+
+
+def test_value_returning_reductions_from_four_threads_on_one_stream():
+    """Each call has its own result cell: threads that share a stream (here the default
+    one, then a created one) must each get their own value back, bit-exact."""
+    import threading
+    rng = np.random.default_rng(21)
+    hosts = [rng.integers(-10**6, 10**6, 40_000 + 1000 * k).astype(np.int64) for k in range(4)]
+    devs = [cuda.to_device(h) for h in hosts]
+    wants = [int(h.sum()) for h in hosts]
+    for stream in (0, cuda.stream()):
+        _say("threads on stream", stream)
+        wrong = []
+
+        def worker(k):
+            for i in range(2000):
+                got = sum_reduce(devs[k], init=i, stream=stream)
+                if int(got) != wants[k] + i:
+                    wrong.append((k, i, int(got)))
+                    return
+
+        threads = [threading.Thread(target=worker, args=(k,)) for k in range(4)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not wrong, wrong
+
+
+def test_per_thread_default_stream_keeps_scratch_per_thread():
+    """cuda.per_thread_default_stream() is one handle but a different stream in every
+    host thread: reductions on it may overlap, so every thread needs scratch of its own."""
+    import threading
+    rng = np.random.default_rng(22)
+    hosts = [rng.integers(-10**6, 10**6, 3_000_000 + 4096 * k).astype(np.int64) for k in range(4)]
+    devs = [cuda.to_device(h) for h in hosts]
+    wants = [int(h.sum()) for h in hosts]
+    wrong = []
+
+    def worker(k):
+        s = cuda.per_thread_default_stream()
+        for i in range(300):
+            got = sum_reduce(devs[k], init=i, stream=s)
+            if int(got) != wants[k] + i:
+                wrong.append((k, i, int(got)))
+                return
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not wrong, wrong

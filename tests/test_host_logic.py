@@ -178,11 +178,56 @@ def test_pending_deallocs_flush_on_bytes(monkeypatch):
     freed = []
     q.add_item(freed.append, "a", 100)
     q.add_item(freed.append, "b", 100)
-    assert len(q) == 2 and q._size == 200          # not above 200 yet
+    assert len(q) == 2 and q.pending_bytes == 200 and q.byte_budget == 200      # not above 200 yet
+    assert (q._size, q._max_pending_bytes) == (200, 200)    # names the reference's own tests read
     q.add_item(freed.append, "c", 1)
-    assert len(q) == 0 and freed == ["a", "b", "c"] and q._size == 0
+    assert len(q) == 0 and freed == ["a", "b", "c"] and q.pending_bytes == 0
     q.add_item(freed.append, "d")                  # unknown size counts as zero
-    assert len(q) == 1 and str(drv._SizeNotSet) == "?"
+    assert len(q) == 1 and q.pending_bytes == 0
+    assert drv._PendingDeallocs().byte_budget == 0     # capacity not known yet
+
+
+def test_pending_deallocs_survive_a_failing_release_and_reentry(monkeypatch):
+    monkeypatch.setattr(config, "CUDA_DEALLOCS_COUNT", 100)
+    q = drv._PendingDeallocs(capacity=1 << 40)
+    freed = []
+
+    def release(h):
+        if h == "bad":
+            raise ValueError("cannot release")
+        if h == "again":
+            q.add_item(freed.append, "late", 8)      # a release that parks another one
+        freed.append(h)
+
+    for h in ("a", "bad", "b", "again"):
+        q.add_item(release, h, 10)
+    with pytest.raises(ValueError):
+        q.clear()
+    assert freed == ["a"] and len(q) == 2 and q.pending_bytes == 20     # the rest is still waiting
+    q.clear()
+    assert freed == ["a", "b", "again"] and len(q) == 1
+    q.clear()
+    assert freed[-1] == "late" and len(q) == 0 and q.pending_bytes == 0
+
+
+def test_pending_deallocs_from_many_threads(monkeypatch):
+    import threading
+    monkeypatch.setattr(config, "CUDA_DEALLOCS_COUNT", 7)
+    q = drv._PendingDeallocs(capacity=1 << 40)
+    freed = []
+
+    def worker(base):
+        for i in range(500):
+            q.add_item(freed.append, base + i, 4)
+
+    threads = [threading.Thread(target=worker, args=(k * 1000,)) for k in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    q.clear()
+    assert sorted(freed) == sorted(k * 1000 + i for k in range(8) for i in range(500))
+    assert q.pending_bytes == 0
 
 
 def test_pending_deallocs_disable_nests():
