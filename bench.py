@@ -6,12 +6,13 @@ on): cuda.reduce float32 sum over 2^28 elements N(0,1), seed 1.  A "step" is one
 full reduction, issued through the public API into a device result slot; inputs
 are resident in HBM before the clock starts.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others]
 
-Other workloads (--workload) report the same line for the remaining benchmark
-configurations: reduce_f32_max, reduce_f64_sum, reduce_i64_sum, transpose_f32,
-transpose_f64, transpose_i16, rng_init, rng_uniform_f32, rng_normal_f64,
-batched_reduce, copy_f32 (counter calibration).
+Without --workload the same line carries an `others` array with every other
+benchmark configuration measured in the same process: reduce_f32_max,
+reduce_f64_sum, reduce_i64_sum, transpose_f32, transpose_f64, transpose_i16,
+rng_init, rng_uniform_f32, rng_normal_f64, batched_reduce.  --workload NAME measures
+just one of them (or copy_f32, the counter calibration kernel) as the headline.
 """
 
 import argparse
@@ -106,8 +107,9 @@ def _cpu_baseline_transpose(shape, dtype):
 
 def _cpu_baseline_rng(name, nthreads=4096):
     """The simulator's RNG: sequential jump chain, then per-thread draws, all in
-    Python over NumPy uint64 scalars, one core, for the 4096 generators the
-    configuration names (about 5 s for the chain, 3 s for the draws)."""
+    Python over NumPy uint64 scalars, one core.  4096 generators are what the
+    configuration names (about 5 s for the chain, 3 s for the draws); the bounded
+    baselines of the `others` array use 1024."""
     from oracle import sim
     from oracle.cref import STATE_DTYPE
     states = np.zeros(nthreads, dtype=STATE_DTYPE)
@@ -245,13 +247,99 @@ def _workload(name, cuda):
     raise SystemExit("unknown workload %s" % name)
 
 
+TRAFFIC_SOURCE = {
+    "reduce_f32_sum": "profiles/reduce_kernel_f32_sum_2p28.txt",
+    "copy_f32": "profiles/copy_flat_f32_2p28.txt",
+    "transpose_f32": "profiles/transpose_packets_f32_16384sq.txt",
+    "rng_uniform_f32": "profiles/xoroshiro_fill_and_init_2p24.txt",
+    "transpose_f64": "profiles/transpose_sheared_f64_12345x6789.txt",
+    "reduce_f32_max": "profiles/hbm_counters_other_workloads.txt",
+    "reduce_f64_sum": "profiles/hbm_counters_other_workloads.txt",
+    "reduce_i64_sum": "profiles/hbm_counters_other_workloads.txt",
+    "transpose_i16": "profiles/hbm_counters_other_workloads.txt",
+    "rng_normal_f64": "profiles/hbm_counters_other_workloads.txt",
+    "rng_init": "profiles/hbm_counters_other_workloads.txt",
+}
+
+OTHER_WORKLOADS = ["reduce_f32_max", "reduce_f64_sum", "reduce_i64_sum", "transpose_f32", "transpose_f64",
+                   "transpose_i16", "rng_init", "rng_uniform_f32", "rng_normal_f64", "batched_reduce"]
+
+
+def _cpu_baseline(name, w, seconds):
+    if name.startswith("reduce_"):
+        is_max = name.endswith("max")
+        return _cpu_baseline_reduce(w["host"], target_seconds=seconds,
+                                    functor=(lambda x, y: max(x, y)) if is_max else (lambda x, y: x + y))
+    if name == "batched_reduce":
+        return _cpu_baseline_reduce(w["host"].reshape(-1), target_seconds=seconds)
+    if name.startswith("transpose_"):
+        return _cpu_baseline_transpose(None, w["dtype"])
+    if name.startswith("rng_"):
+        # the sequential jump chain costs about 1.2 ms per generator
+        return _cpu_baseline_rng(name, nthreads=4096 if seconds >= 8 else 1024)
+    return None
+
+
+def measure(cuda, name, steps, warmup, cpu_seconds):
+    """One workload: `warmup` untimed steps, `steps` timed ones between device-wide
+    synchronisations (wall clock -> value), the same number again between a HIP
+    event pair on the launch stream (-> roofline), and the CPU baseline beside it
+    (cpu_seconds = 0: none)."""
+    w = _workload(name, cuda)
+    stream, step = w["stream"], w["step"]
+    for i in range(warmup):
+        step(i)
+    stream.synchronize()
+    cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    stream.synchronize()
+    cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / steps * 1e3
+    gbs = w["algo_bytes"] / (ms_per_step * 1e-3) / 1e9
+
+    roofline = None
+    if "calls_per_step" not in w:
+        launch_ms = _event_timed_launches(cuda, stream, step, steps)
+        achieved = w["algo_bytes"] / (launch_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(name),
+                    # `traffic` was not measured in this run: it is the rocprofv3 counter
+                    # figure recorded in the named file for this workload
+                    "traffic_source": TRAFFIC_SOURCE.get(name),
+                    "kernel": w["kernel"], "algorithmic_bytes_per_launch": w["algo_bytes"],
+                    "launch_us_avg": round(launch_ms * 1e3, 2), "launches_timed": steps}
+    cpu = _cpu_baseline(name, w, cpu_seconds) if cpu_seconds > 0 else None
+    out = {"name": name, "workload": w["desc"], "dtype": w["dtype"], "value": round(gbs, 1), "unit": "GB/s",
+           "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 5),
+           "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+           "units_per_s": round(w["units"] / (ms_per_step * 1e-3), 1),
+           "roofline": roofline, "cpu_baseline": cpu}
+    if "calls_per_step" in w:
+        out["us_per_call"] = round(ms_per_step * 1e3 / w["calls_per_step"], 3)
+    return out
+
+
+def _release_device_memory(cuda):
+    import gc
+    gc.collect()
+    ctx = cuda.current_context()
+    ctx.memory_manager.deallocations.clear()
+    ctx.deallocations.clear()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="reduce_f32_sum")
+    ap.add_argument("--workload", default=None,
+                    help="measure only this workload (default: the headline workload, then every other "
+                         "configuration in an `others` array)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-others", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
@@ -260,57 +348,32 @@ def main():
     import numba_cuda_amd as cuda
     if not cuda.is_available():
         raise SystemExit("no GPU / HIP library: %s" % cuda.cuda_error())
-    w = _workload(args.workload, cuda)
-    stream, step = w["stream"], w["step"]
 
-    for i in range(args.warmup):
-        step(i)
-    stream.synchronize()
-    cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
-    stream.synchronize()
-    cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall / args.steps * 1e3
-    gbs = w["algo_bytes"] / (ms_per_step * 1e-3) / 1e9
-
-    roofline = None
-    if "calls_per_step" not in w:
-        launch_ms = _event_timed_launches(cuda, stream, step, args.steps)
-        achieved = w["algo_bytes"] / (launch_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(args.workload),
-                    "kernel": w["kernel"], "algorithmic_bytes_per_launch": w["algo_bytes"],
-                    "launch_us_avg": round(launch_ms * 1e3, 2), "launches_timed": args.steps}
-
-    cpu = None
-    if not args.no_cpu_baseline:
-        name = args.workload
-        if name.startswith("reduce_"):
-            is_max = name.endswith("max")
-            cpu = _cpu_baseline_reduce(w["host"], functor=(lambda x, y: max(x, y)) if is_max else (lambda x, y: x + y))
-        elif name == "batched_reduce":
-            cpu = _cpu_baseline_reduce(w["host"].reshape(-1))
-        elif name.startswith("transpose_"):
-            cpu = _cpu_baseline_transpose(None, w["dtype"])
-        elif name.startswith("rng_"):
-            cpu = _cpu_baseline_rng(name)
-
+    name = args.workload or "reduce_f32_sum"
+    head = measure(cuda, name, args.steps, args.warmup, 0 if args.no_cpu_baseline else 12.0)
     line = {
         "metric": "achieved HBM GB/s (% of 8 TB/s) for cuda.reduce fp32 sum at 2^28 elems"
-        if args.workload == "reduce_f32_sum" else "achieved HBM GB/s for " + args.workload,
-        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
-        "config": {"workload": w["desc"], "name": args.workload},
-        "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
-        "units_per_s": round(w["units"] / (ms_per_step * 1e-3), 1),
-        "roofline": roofline, "cpu_baseline": cpu,
+        if name == "reduce_f32_sum" else "achieved HBM GB/s for " + name,
+        "value": head["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": head["workload"], "name": name},
+        "pct_of_hbm_peak": head["pct_of_hbm_peak"], "units_per_s": head["units_per_s"],
+        "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"],
     }
-    if "calls_per_step" in w:
-        line["us_per_call"] = round(ms_per_step * 1e3 / w["calls_per_step"], 3)
+    if "us_per_call" in head:
+        line["us_per_call"] = head["us_per_call"]
+
+    if args.workload is None and not args.no_others:
+        # every other benchmark configuration, in this same process: fewer steps, and a CPU
+        # baseline bounded to about two seconds each
+        others = []
+        for other in OTHER_WORKLOADS:
+            _release_device_memory(cuda)
+            steps, warmup = (3, 1) if other == "batched_reduce" else (min(args.steps, 50), min(args.warmup, 5))
+            print("bench: %s ..." % other, file=sys.stderr, flush=True)
+            others.append(measure(cuda, other, steps, warmup, 0 if args.no_cpu_baseline else 2.0))
+        line["others"] = others
     print(json.dumps(line))
 
 
