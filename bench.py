@@ -184,7 +184,7 @@ def _workload(name, cuda):
         return dict(desc="transpose %s %dx%d, seed 2" % (host.dtype.name, host.shape[0], host.shape[1]),
                     dtype=host.dtype.name, algo_bytes=2 * host.nbytes, units=host.size, step=step,
                     stream=stream, host=None, keep=(src, dst),
-                    kernel={"transpose_f32": "transpose_packets<4, true>", "transpose_f64": "transpose_sheared<8>",
+                    kernel={"transpose_f32": "transpose_packets<4, true>", "transpose_f64": "transpose_sheared<RingCfg<8, 128, 32, 4, 256, 1>>",
                             "transpose_i16": "transpose_packets<2, true>"}[name])
     if name.startswith("rng_"):
         n = 2**24

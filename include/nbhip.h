@@ -38,7 +38,8 @@ enum nbh_dtype {
     NBH_U8 = 4, NBH_U16 = 5, NBH_U32 = 6, NBH_U64 = 7,
     NBH_F32 = 8, NBH_F64 = 9,
     NBH_C64 = 10, NBH_C128 = 11,   /* complex: pairs (re, im) of float32 / float64; ADD and MUL only */
-    NBH_DTYPE_COUNT = 12
+    NBH_F16 = 12,                  /* IEEE binary16; accumulated in binary16, one rounding per operation */
+    NBH_DTYPE_COUNT = 13
 };
 
 /* binary operators understood by nbh_reduce.  Semantics are those the reference's
@@ -238,6 +239,17 @@ int nbh_xoro_uniform_f32(void *states, int64_t nstates, float *out, int64_t coun
 int nbh_xoro_uniform_f64(void *states, int64_t nstates, double *out, int64_t count, nbh_stream_t stream);
 int nbh_xoro_normal_f32(void *states, int64_t nstates, float *out, int64_t count, nbh_stream_t stream);
 int nbh_xoro_normal_f64(void *states, int64_t nstates, double *out, int64_t count, nbh_stream_t stream);
+
+/* random.py:96-238 the per-generator functions xoroshiro128p_next / _jump /
+ * _uniform_float32 / _uniform_float64 / _normal_float32 / _normal_float64 applied to ONE
+ * generator of a device-resident state array (the reference's simulator lets host code
+ * call them on the array create_xoroshiro128p_states returned).  `state` points to the
+ * generator's 16-byte record in device memory and is advanced in place; the value goes
+ * to `out`, 8-byte aligned memory the device can address (uint64 for NEXT, float /
+ * double for the draws; unused and may be NULL for JUMP).  Same bits as the bulk calls. */
+enum nbh_xoro_kind { NBH_XORO_NEXT = 0, NBH_XORO_JUMP = 1, NBH_XORO_UNIFORM_F32 = 2, NBH_XORO_UNIFORM_F64 = 3,
+                     NBH_XORO_NORMAL_F32 = 4, NBH_XORO_NORMAL_F64 = 5 };
+int nbh_xoro_one(void *state, int kind, void *out, nbh_stream_t stream);
 
 #ifdef __cplusplus
 }

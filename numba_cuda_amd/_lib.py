@@ -75,12 +75,14 @@ SIGNATURES = {
     "nbh_xoro_uniform_f64": (c_int, [c_vp, c_i64, c_vp, c_i64, c_vp]),
     "nbh_xoro_normal_f32": (c_int, [c_vp, c_i64, c_vp, c_i64, c_vp]),
     "nbh_xoro_normal_f64": (c_int, [c_vp, c_i64, c_vp, c_i64, c_vp]),
+    "nbh_xoro_one": (c_int, [c_vp, c_int, c_vp, c_vp]),
 }
 
 # enum nbh_dtype / enum nbh_op
 DTYPE_CODES = {"int8": 0, "int16": 1, "int32": 2, "int64": 3,
                "uint8": 4, "uint16": 5, "uint32": 6, "uint64": 7,
-               "float32": 8, "float64": 9, "complex64": 10, "complex128": 11}
+               "float32": 8, "float64": 9, "complex64": 10, "complex128": 11,
+               "float16": 12}
 OP_CODES = {"add": 0, "mul": 1, "max": 2, "min": 3, "and": 4, "or": 5, "xor": 6}
 
 # hipError_t values the Python layer branches on

@@ -68,8 +68,13 @@ template <typename R> __device__ __forceinline__ Cplx<R> operator*(Cplx<R> a, Cp
 }
 template <typename T> struct IsCplx : std::false_type {};
 template <typename R> struct IsCplx<Cplx<R>> : std::true_type {};
+// float16 elements: the accumulator is a half too, every operation rounds to binary16
+// (what the reference's JIT emits for `a + b` on float16 operands)
+using Half = _Float16;
+// real floating point, binary16 included
+template <typename T> struct IsReal : std::integral_constant<bool, std::is_floating_point<T>::value || std::is_same<T, Half>::value> {};
 // real or complex floating point: the accumulator is the element type itself
-template <typename T> struct IsInexact : std::integral_constant<bool, std::is_floating_point<T>::value || IsCplx<T>::value> {};
+template <typename T> struct IsInexact : std::integral_constant<bool, IsReal<T>::value || IsCplx<T>::value> {};
 
 // ---- operators -----------------------------------------------------------------
 struct OpAdd {
@@ -119,12 +124,12 @@ template <typename T, typename Op> __device__ __forceinline__ typename AccOf<T, 
         return (A) ~(A)0;
     else if constexpr (std::is_same<Op, OpMul>::value)
         return A(1);
+    else if constexpr (IsReal<T>::value)
+        return std::is_same<Op, OpMax>::value ? A(-__builtin_huge_valf()) : A(__builtin_huge_valf());
     else if constexpr (std::is_same<Op, OpMax>::value)
-        return std::is_floating_point<T>::value ? A(-std::numeric_limits<T>::infinity())
-                                                : A(std::numeric_limits<T>::lowest());
+        return A(std::numeric_limits<T>::lowest());
     else
-        return std::is_floating_point<T>::value ? A(std::numeric_limits<T>::infinity())
-                                                : A(std::numeric_limits<T>::max());
+        return A(std::numeric_limits<T>::max());
 }
 
 // ---- wavefront / workgroup folding -----------------------------------------------
@@ -135,7 +140,10 @@ template <int CTRL> __device__ __forceinline__ uint32_t dpp_move(uint32_t v)
 
 template <typename A, int CTRL> __device__ __forceinline__ A dpp(A v)
 {
-    if constexpr (sizeof(A) == 4) {
+    if constexpr (sizeof(A) == 2) {
+        uint16_t b = __builtin_bit_cast(uint16_t, v);
+        return __builtin_bit_cast(A, (uint16_t)dpp_move<CTRL>(b));
+    } else if constexpr (sizeof(A) == 4) {
         uint32_t b = __builtin_bit_cast(uint32_t, v);
         return __builtin_bit_cast(A, dpp_move<CTRL>(b));
     } else if constexpr (sizeof(A) == 8) {
@@ -144,7 +152,7 @@ template <typename A, int CTRL> __device__ __forceinline__ A dpp(A v)
         uint32_t hi = dpp_move<CTRL>((uint32_t)(b >> 32));
         return __builtin_bit_cast(A, ((uint64_t)hi << 32) | lo);
     } else {
-        static_assert(sizeof(A) == 16, "accumulators are 4, 8 or 16 bytes");
+        static_assert(sizeof(A) == 16, "accumulators are 2, 4, 8 or 16 bytes");
         nbh_u32x4 b = __builtin_bit_cast(nbh_u32x4, v);
 #pragma unroll
         for (int k = 0; k < 4; ++k)
@@ -155,7 +163,10 @@ template <typename A, int CTRL> __device__ __forceinline__ A dpp(A v)
 
 template <typename A> __device__ __forceinline__ A read_lane(A v, int lane)
 {
-    if constexpr (sizeof(A) == 4) {
+    if constexpr (sizeof(A) == 2) {
+        uint16_t b = __builtin_bit_cast(uint16_t, v);
+        return __builtin_bit_cast(A, (uint16_t)__builtin_amdgcn_readlane((int)b, lane));
+    } else if constexpr (sizeof(A) == 4) {
         uint32_t b = __builtin_bit_cast(uint32_t, v);
         return __builtin_bit_cast(A, (uint32_t)__builtin_amdgcn_readlane((int)b, lane));
     } else if constexpr (sizeof(A) == 8) {
@@ -200,11 +211,28 @@ template <typename A, typename Op> __device__ __forceinline__ A block_fold(A v, 
 // 8-byte words; each word is one atomic store, the ticket is drawn after all of them
 // have been acknowledged).
 template <typename A> struct WordsOf {
-    using Word = typename std::conditional<sizeof(A) == 4, uint32_t, uint64_t>::type;
-    static constexpr int kWords = (int)(sizeof(A) / sizeof(Word));
+    using Word = typename std::conditional<sizeof(A) <= 4, uint32_t, uint64_t>::type;
+    static constexpr int kWords = sizeof(A) <= 4 ? 1 : (int)(sizeof(A) / sizeof(Word));
     struct Image {
         Word w[kWords];
     };
+    static __device__ __forceinline__ Image pack(A v)
+    {
+        if constexpr (sizeof(A) == 2) {  // a half travels in the low 16 bits of a word
+            Image img;
+            img.w[0] = __builtin_bit_cast(uint16_t, v);
+            return img;
+        } else {
+            return __builtin_bit_cast(Image, v);
+        }
+    }
+    static __device__ __forceinline__ A unpack(Image img)
+    {
+        if constexpr (sizeof(A) == 2)
+            return __builtin_bit_cast(A, (uint16_t)img.w[0]);
+        else
+            return __builtin_bit_cast(A, img);
+    }
 };
 
 // ---- the kernel ------------------------------------------------------------------
@@ -302,7 +330,7 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
 
     Word *partials = reinterpret_cast<Word *>(partials_raw);
     if (tid == 0) {
-        const Image img = __builtin_bit_cast(Image, total);
+        const Image img = WordsOf<A>::pack(total);
         Word before[kWords];
 #pragma unroll
         for (int w = 0; w < kWords; ++w)
@@ -329,7 +357,7 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
         for (int w = 0; w < kWords; ++w)
             img.w[w] = __hip_atomic_load(&partials[(int64_t)k * kWords + w], __ATOMIC_RELAXED,
                                          __HIP_MEMORY_SCOPE_AGENT);
-        fin = Op::apply(fin, __builtin_bit_cast(A, img));
+        fin = Op::apply(fin, WordsOf<A>::unpack(img));
     }
     fin = block_fold<A, Op>(fin, lds);
     if (tid == 0) {
@@ -439,6 +467,7 @@ int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, 
     case NBH_U64: return launch_op<uint64_t>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_F32: return launch_op<float>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_F64: return launch_op<double>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_F16: return launch_op<Half>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_C64: return launch_op_complex<Cplx<float>>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_C128: return launch_op_complex<Cplx<double>>(op, in, n, in_stride, init, out, scratch, s);
     default: return (int)hipErrorInvalidValue;

@@ -100,14 +100,14 @@ __device__ __forceinline__ void move_block(const char *__restrict__ in, char *__
     }
 }
 
-template <int E, bool NT>
-__global__ __launch_bounds__(64 * ShapeOf<E>::WR * ShapeOf<E>::WC) void transpose_packets(
+template <int E, bool NT, typename Shape = ShapeOf<E>>
+__global__ __launch_bounds__(64 * Shape::WR * Shape::WC) void transpose_packets(
     const char *__restrict__ in, char *__restrict__ out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
     int64_t tiles_r)
 {
     constexpr int V = 16 / E;
     constexpr int WT = 8 * V;  // wavefront tile edge, in items
-    constexpr int WR = ShapeOf<E>::WR, WC = ShapeOf<E>::WC, REP = ShapeOf<E>::REP;
+    constexpr int WR = Shape::WR, WC = Shape::WC, REP = Shape::REP;
     constexpr int TR = WT * WR * REP, TC = WT * WC;
 
     // consecutive workgroups go down the input rows = along the output rows
@@ -145,26 +145,38 @@ __global__ __launch_bounds__(64 * ShapeOf<E>::WR * ShapeOf<E>::WC) void transpos
 // Measured: float64 12345 x 6789 4.0 -> 5.1 TB/s, float32 16388 x 16384 4.1 -> 5.0.
 // One-byte items stay with the packet kernel: gathering 16 single bytes from the ring
 // per store costs more than the straddling does (2.5 against 3.2 TB/s).
-template <int E> struct ShearOf;   // RING must be a power of two
-template <> struct ShearOf<2> { static constexpr int RING = 256, TC = 64, PAD = 2; };
-template <> struct ShearOf<4> { static constexpr int RING = 128, TC = 32, PAD = 2; };
-template <> struct ShearOf<8> { static constexpr int RING = 64, TC = 32, PAD = 4; };
-template <> struct ShearOf<16> { static constexpr int RING = 32, TC = 32, PAD = 1; };
-constexpr int kStripSteps = 8;  // steps of TR rows per workgroup
+// Shape of the ring kernel.  RING (a power of two) rows of TC columns, THREADS lanes,
+// STEPS steps of TR = RING - L rows per workgroup.
+template <int E_, int RING_, int TC_, int PAD_, int THREADS_, int STEPS_> struct RingCfg {
+    static constexpr int E = E_, RING = RING_, TC = TC_, PAD = PAD_, THREADS = THREADS_, STEPS = STEPS_;
+};
+// Measured on MI355X (TB/s of algorithmic traffic, ring 64 rows x 8 steps -> these shapes):
+// float64 12345 x 6789 5.07 -> 5.44, float32 16388 x 16384 5.10 -> 5.75, 16385^2 5.09 -> 5.32,
+// int16 8193 x 32769 4.40 -> 5.04, 16-byte items 8193^2 5.18 -> 5.86.  Tall tiles win (long
+// runs of every output row are written by one workgroup at one time) and so do short
+// strips: with one step per workgroup there are more, shorter workgroups in flight and
+// the L rows above a strip, read a second time, cost less than the lost overlap did.
+template <int E> struct ShearOf;
+template <> struct ShearOf<2> { using type = RingCfg<2, 256, 64, 2, 256, 2>; };
+template <> struct ShearOf<4> { using type = RingCfg<4, 256, 64, 4, 512, 1>; };
+template <> struct ShearOf<8> { using type = RingCfg<8, 128, 32, 4, 256, 1>; };
+template <> struct ShearOf<16> { using type = RingCfg<16, 64, 32, 1, 256, 1>; };
 
-template <int E>
-__global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__restrict__ in, char *__restrict__ out,
-                                                               int64_t rows, int64_t cols, int64_t in_s0,
-                                                               int64_t out_s0, int64_t strips_r, bool by_xcd)
+template <typename Cfg>
+__global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__restrict__ in, char *__restrict__ out,
+                                                                   int64_t rows, int64_t cols, int64_t in_s0,
+                                                                   int64_t out_s0, int64_t strips_r, bool by_xcd)
 {
+    constexpr int E = Cfg::E;
     using Item = typename ItemOf<E>::type;
     constexpr int V = 16 / E;    // items per packet
     constexpr int L = 128 / E;   // items per cache line
-    constexpr int RING = ShearOf<E>::RING, TC = ShearOf<E>::TC;
+    constexpr int RING = Cfg::RING, TC = Cfg::TC, kThr = Cfg::THREADS;
     constexpr int TR = RING - L;
-    constexpr int PPR = TC / V;  // packets per tile row
+    constexpr int PPR = TC / V;     // packets per tile row
     constexpr int NL = TR / L + 2;  // lines of one output row a step can touch, at most
-    __shared__ Item ring[RING][TC + ShearOf<E>::PAD];
+    static_assert((RING & (RING - 1)) == 0 && TR > 0, "ring depth");
+    __shared__ Item ring[RING][TC + Cfg::PAD];
 
     const int tid = threadIdx.x;
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  When a
@@ -180,15 +192,15 @@ __global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__rest
     const int64_t tile_c = logical / strips_r;
     const int64_t strip = logical % strips_r;
     const int64_t C0 = tile_c * TC;
-    const int64_t strip_begin = strip * (int64_t)(kStripSteps * TR);
-    int64_t strip_end = strip_begin + (int64_t)kStripSteps * TR;
+    const int64_t strip_begin = strip * (int64_t)(Cfg::STEPS * TR);
+    int64_t strip_end = strip_begin + (int64_t)Cfg::STEPS * TR;
     const bool last_strip = strip == strips_r - 1;
     if (last_strip)
         strip_end = rows;
 
     // A step's rows travel global -> registers -> ring, so that the loads of the next
     // step are already in flight while this step's rows are being written out.
-    constexpr int NP = (RING * PPR + kThreads - 1) / kThreads;  // packets per thread, at most
+    constexpr int NP = (RING * PPR + kThr - 1) / kThr;  // packets per thread, at most
     union Pack {
         u32x4 pk;
         Item it[V];
@@ -199,7 +211,7 @@ __global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__rest
         const int count = (int)(to - from) * PPR;
 #pragma unroll
         for (int k = 0; k < NP; ++k) {
-            const int idx = tid + k * kThreads;
+            const int idx = tid + k * kThr;
             if (idx >= count)
                 break;
             const int64_t gr = from + idx / PPR;
@@ -220,7 +232,7 @@ __global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__rest
         const int count = (int)(to - from) * PPR;
 #pragma unroll
         for (int k = 0; k < NP; ++k) {
-            const int idx = tid + k * kThreads;
+            const int idx = tid + k * kThr;
             if (idx >= count)
                 break;
             const int64_t gr = from + idx / PPR;
@@ -246,8 +258,8 @@ __global__ __launch_bounds__(kThreads) void transpose_sheared(const char *__rest
         if (next < strip_end)
             fetch(next, next_end);
         // eight lanes per 128-byte line of output; a pass of the workgroup covers
-        // kThreads / 8 lines, neighbouring output rows first
-        for (int w = tid >> 3; w < TC * NL; w += kThreads / 8) {
+        // kThr / 8 lines, neighbouring output rows first
+        for (int w = tid >> 3; w < TC * NL; w += kThr / 8) {
             const int lc = w % TC, k = w / TC;
             const int64_t c = C0 + lc;
             if (c >= cols)
@@ -387,12 +399,12 @@ __global__ __launch_bounds__(kThreads) void transpose_strided(const char *__rest
     }
 }
 
-template <int E>
+template <int E, typename Shape = ShapeOf<E>>
 int launch_packets(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
                    hipStream_t stream)
 {
     constexpr int WT = 8 * (16 / E);
-    constexpr int TR = WT * ShapeOf<E>::WR * ShapeOf<E>::REP, TC = WT * ShapeOf<E>::WC;
+    constexpr int TR = WT * Shape::WR * Shape::REP, TC = WT * Shape::WC;
     const int64_t tiles_r = (rows + TR - 1) / TR;
     const int64_t tiles_c = (cols + TC - 1) / TC;
     const int64_t tiles = tiles_r * tiles_c;
@@ -400,13 +412,31 @@ int launch_packets(const void *in, void *out, int64_t rows, int64_t cols, int64_
         return (int)hipErrorInvalidValue;
     // stream past the caches only if every row of both arrays starts on a 128-byte line
     const uint64_t mix = (uint64_t)(uintptr_t)in | (uint64_t)(uintptr_t)out | (uint64_t)in_s0 | (uint64_t)out_s0;
-    const dim3 grid((unsigned)tiles), block(64 * ShapeOf<E>::WR * ShapeOf<E>::WC);
+    const dim3 grid((unsigned)tiles), block(64 * Shape::WR * Shape::WC);
     if (mix % 128 == 0)
-        hipLaunchKernelGGL((transpose_packets<E, true>), grid, block, 0, stream, (const char *)in, (char *)out, rows,
-                           cols, in_s0, out_s0, tiles_r);
+        hipLaunchKernelGGL((transpose_packets<E, true, Shape>), grid, block, 0, stream, (const char *)in, (char *)out,
+                           rows, cols, in_s0, out_s0, tiles_r);
     else
-        hipLaunchKernelGGL((transpose_packets<E, false>), grid, block, 0, stream, (const char *)in, (char *)out, rows,
-                           cols, in_s0, out_s0, tiles_r);
+        hipLaunchKernelGGL((transpose_packets<E, false, Shape>), grid, block, 0, stream, (const char *)in, (char *)out,
+                           rows, cols, in_s0, out_s0, tiles_r);
+    return nbh_launch_status();
+}
+
+template <typename Cfg>
+int launch_sheared_cfg(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
+                       hipStream_t stream)
+{
+    constexpr int E = Cfg::E;
+    constexpr int TR = Cfg::RING - 128 / E;
+    const int64_t strips_r = (rows + (int64_t)Cfg::STEPS * TR - 1) / ((int64_t)Cfg::STEPS * TR);
+    const int64_t tiles_c = (cols + Cfg::TC - 1) / Cfg::TC;
+    const int64_t blocks = strips_r * tiles_c;
+    if (blocks > 0x7fffffffLL)
+        return (int)hipErrorInvalidValue;
+    const bool ragged_in = (((uint64_t)(uintptr_t)in | (uint64_t)in_s0) % 128) != 0;
+    const bool by_xcd = ragged_in && Cfg::TC * E <= 128;
+    hipLaunchKernelGGL((transpose_sheared<Cfg>), dim3((unsigned)blocks), dim3(Cfg::THREADS), 0, stream,
+                       (const char *)in, (char *)out, rows, cols, in_s0, out_s0, strips_r, by_xcd);
     return nbh_launch_status();
 }
 
@@ -414,17 +444,7 @@ template <int E>
 int launch_sheared(const void *in, void *out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
                    hipStream_t stream)
 {
-    constexpr int TR = ShearOf<E>::RING - 128 / E;
-    const int64_t strips_r = (rows + (int64_t)kStripSteps * TR - 1) / ((int64_t)kStripSteps * TR);
-    const int64_t tiles_c = (cols + ShearOf<E>::TC - 1) / ShearOf<E>::TC;
-    const int64_t blocks = strips_r * tiles_c;
-    if (blocks > 0x7fffffffLL)
-        return (int)hipErrorInvalidValue;
-    const bool ragged_in = (((uint64_t)(uintptr_t)in | (uint64_t)in_s0) % 128) != 0;
-    const bool by_xcd = ragged_in && ShearOf<E>::TC * E <= 128;
-    hipLaunchKernelGGL((transpose_sheared<E>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, (const char *)in,
-                       (char *)out, rows, cols, in_s0, out_s0, strips_r, by_xcd);
-    return nbh_launch_status();
+    return launch_sheared_cfg<typename ShearOf<E>::type>(in, out, rows, cols, in_s0, out_s0, stream);
 }
 
 template <int G>

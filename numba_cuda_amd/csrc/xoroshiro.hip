@@ -823,9 +823,74 @@ int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t 
     return nbh_launch_status();
 }
 
+// ---- one generator at a time --------------------------------------------------------
+// What the per-generator functions of the Python layer run when the states live on the
+// device: one lane, the same draw routines as the bulk kernels (hence the same bits).
+__global__ __launch_bounds__(64) void one_generator_kernel(uint64_t *__restrict__ state, int kind,
+                                                           void *__restrict__ out,
+                                                           const bm::LogTable *__restrict__ log_table)
+{
+    if (threadIdx.x != 0)
+        return;
+    uint64_t s0 = state[0], s1 = state[1];
+    switch (kind) {
+    case NBH_XORO_NEXT:
+        *static_cast<uint64_t *>(out) = next_d(s0, s1);
+        break;
+    case NBH_XORO_JUMP: {
+        // random.py:118-142: XOR together the states reached after k steps for every set
+        // bit k of the 128-bit jump polynomial (= 2^64 steps)
+        const uint64_t poly[2] = {0xBEAC0467EBA5FACBull, 0xD86B048B86AA9922ull};
+        uint64_t j0 = 0, j1 = 0;
+        for (int w = 0; w < 2; ++w)
+            for (int b = 0; b < 64; ++b) {
+                if ((poly[w] >> b) & 1) {
+                    j0 ^= s0;
+                    j1 ^= s1;
+                }
+                (void)next_d(s0, s1);
+            }
+        s0 = j0;
+        s1 = j1;
+        break;
+    }
+    case NBH_XORO_UNIFORM_F32:
+        *static_cast<float *>(out) = UniformF32::draw(s0, s1);
+        break;
+    case NBH_XORO_UNIFORM_F64:
+        *static_cast<double *>(out) = UniformF64::draw(s0, s1);
+        break;
+    case NBH_XORO_NORMAL_F32:
+        *static_cast<float *>(out) = NormalF32::draw(s0, s1, log_table);
+        break;
+    default:
+        *static_cast<double *>(out) = NormalF64::draw(s0, s1, log_table);
+        break;
+    }
+    state[0] = s0;
+    state[1] = s1;
+}
+
 }  // namespace
 
 extern "C" {
+
+int nbh_xoro_one(void *state, int kind, void *out, nbh_stream_t stream)
+{
+    if (!state || ((uintptr_t)state) % 16 != 0 || kind < NBH_XORO_NEXT || kind > NBH_XORO_NORMAL_F64)
+        return (int)hipErrorInvalidValue;
+    if (kind != NBH_XORO_JUMP && (!out || ((uintptr_t)out) % 8 != 0))
+        return (int)hipErrorInvalidValue;
+    const bm::LogTable *log_table = nullptr;
+    if (kind == NBH_XORO_NORMAL_F32 || kind == NBH_XORO_NORMAL_F64)
+        if (int rc = device_log_table(&log_table))
+            return rc;
+    hipLaunchKernelGGL(one_generator_kernel, dim3(1), dim3(64), 0, nbh_hip_stream(stream), (uint64_t *)state, kind,
+                       out, log_table);
+    const int rc = nbh_launch_status();
+    nbh_pool_note_stream(nbh_hip_stream(stream));
+    return rc;
+}
 
 int nbh_xoro_init_states(void *states, int64_t n, uint64_t seed, uint64_t subsequence_start, nbh_stream_t stream)
 {

@@ -4,7 +4,8 @@ Drop-in for numba_cuda/numba/cuda/kernels/reduction.py:169-265.  The reference
 JIT-compiles the Python functor into a three-launch tree reduction; here the
 functor is *recognised* as one of the operators that have hand-written HIP
 kernels (a + b, a * b, max(a, b), min(a, b), and a & b, a | b, a ^ b on integers) and a single launch of
-nbh_reduce does the work.  Anything else raises NotImplementedError - there is
+nbh_reduce does the work.  Element types: the integers, booleans, float16 (accumulated in
+float16, as the reference's JIT does), float32, float64, complex64 and complex128.  Anything else raises NotImplementedError - there is
 no slower path to fall back to.
 """
 
@@ -180,16 +181,22 @@ class Reduce:
             except TypeError:
                 pass
         self._opcode = _lib.OP_CODES[self._op]
-        self._codes = {}    # dtype -> element code, filled once the pairing with the operator is checked
+        self._codes = {}    # dtype -> (operator code, element code), filled once the pairing is checked
 
-    def _element_code(self, dtype):
+    def _codes_for(self, dtype):
+        """(operator code, element code) nbh_reduce is called with for arrays of `dtype`."""
+        opcode = self._opcode
         if dtype == _BOOL:
-            # one byte holding 0 or 1: and / or / xor / max / min of those are again 0 or 1,
-            # so the uint8 kernels do (sums and products of booleans are integers in the
-            # reference and are not offered here)
-            if self._op in ("add", "mul"):
-                raise NotImplementedError("Reduce does not add or multiply booleans; use a & b, a | b, a ^ b, max or min")
-            return _DTYPE_CODE[np.dtype(np.uint8)]
+            # One byte holding 0 or 1, reduced by the uint8 kernels.  and / or / xor / max /
+            # min of such bytes are again 0 or 1.  `a + b` and `a * b` are typed int64 by
+            # the reference's JIT and converted back with `!= 0` wherever the kernels store
+            # them into their boolean arrays (kernels/reduction.py:32-37, :96), which makes
+            # the sum "any is true" and the product "all are true": the or / and kernels.
+            if self._op == "add":
+                opcode = _lib.OP_CODES["or"]
+            elif self._op == "mul":
+                opcode = _lib.OP_CODES["and"]
+            return opcode, _DTYPE_CODE[np.dtype(np.uint8)]
         code = _DTYPE_CODE.get(dtype)
         if code is None:
             raise NotImplementedError("Reduce does not support dtype %s" % dtype)
@@ -199,7 +206,7 @@ class Reduce:
         if dtype.kind not in "iu" and self._op in ("and", "or", "xor"):
             # the reference fails at compile time too: no bitwise operators on floating point
             raise TypeError("bitwise %s is not defined for %s" % (self._op, dtype))
-        return code
+        return opcode, code
 
     def __call__(self, arr, size=None, res=None, init=0, stream=0):
         """Full reduction of `arr`.
@@ -220,9 +227,10 @@ class Reduce:
         if arr.size < 1:
             return dtype.type(init)          # `res` is left untouched, as in the reference
 
-        code = self._codes.get(dtype)
-        if code is None:
-            code = self._codes[dtype] = self._element_code(dtype)
+        codes = self._codes.get(dtype)
+        if codes is None:
+            codes = self._codes[dtype] = self._codes_for(dtype)
+        opcode, code = codes
 
         ctx = devices.get_context()
         if not _driver.is_device_memory(arr):
@@ -236,7 +244,7 @@ class Reduce:
         if res is not None:
             if res.dtype != dtype:
                 raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
-            rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size,
+            rc = drv.lib.nbh_reduce(opcode, code, arr.device_ctypes_pointer.value, arr.size,
                                     arr.strides[0], init_ptr, res.device_ctypes_pointer.value,
                                     scratch_ptr, scratch_bytes, hstream or None)
             if rc:
@@ -248,7 +256,7 @@ class Reduce:
         # stream and reads the cell - no copy back.
         cell = ctx.take_result_cell()
         try:
-            rc = drv.lib.nbh_reduce(self._opcode, code, arr.device_ctypes_pointer.value, arr.size,
+            rc = drv.lib.nbh_reduce(opcode, code, arr.device_ctypes_pointer.value, arr.size,
                                     arr.strides[0], init_ptr, cell[0],
                                     scratch_ptr, scratch_bytes, hstream or None)
             if rc:

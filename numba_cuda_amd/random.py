@@ -10,8 +10,11 @@ Differences in mechanism, not in results:
     generator t, `count` values into out[t*count + i] - the layout of the
     reference's own test kernels (tests/cudapy/test_random.py:29-52)
   * the scalar functions `xoroshiro128p_next(states, index)` etc. keep their
-    reference meaning on HOST state arrays (the reference's functions are also
-    CPU-callable); device arrays are refused with a pointer to the bulk call.
+    reference meaning when called from host code, on host state arrays and on the
+    device array create_xoroshiro128p_states returned alike (the reference's
+    simulator allows both): on a device array the one generator is stepped by a
+    one-lane kernel running the same routines as the bulk draws, and the value
+    comes back through a cell of device-mapped host memory.
 """
 
 import math
@@ -110,18 +113,50 @@ def xoroshiro128p_fill_normal(states, out, count=None, stream=0):
     return xoroshiro128p_fill(states, out, count, NORMAL, stream)
 
 
-# ---- scalar functions on host state arrays (reference semantics, random.py:62-238) ----
+# ---- scalar functions (reference semantics, random.py:62-238) --------------------------
 
-def _host_states(states):
-    if _driver.is_device_memory(states):
-        raise TypeError("per-generator draws need a host array of states; on the device use "
-                        "xoroshiro128p_fill(states, out, count, distribution)")
-    return states
+_ONE_NEXT, _ONE_JUMP, _ONE_UNIFORM_F32, _ONE_UNIFORM_F64, _ONE_NORMAL_F32, _ONE_NORMAL_F64 = range(6)   # nbh_xoro_kind
+_ONE_RESULT = {_ONE_NEXT: np.dtype(np.uint64), _ONE_UNIFORM_F32: np.dtype(np.float32),
+               _ONE_UNIFORM_F64: np.dtype(np.float64), _ONE_NORMAL_F32: np.dtype(np.float32),
+               _ONE_NORMAL_F64: np.dtype(np.float64)}
+
+
+def _record_address(states, index):
+    """Device address of generator `index` of a device-resident state array."""
+    if states.ndim != 1 or states.dtype.itemsize != 16:
+        raise TypeError("states must be a 1D array of xoroshiro128p_dtype")
+    index = int(index)
+    n = states.size
+    if not -n <= index < n:
+        raise IndexError("index %d is out of bounds for %d generator states" % (index, n))
+    return states.device_ctypes_pointer.value + (index % n) * states.strides[0]
+
+
+def _on_device(states, index, kind):
+    """Run one per-generator function on generator `index` of a device array and
+    return its value (None for the jump)."""
+    ctx = devices.get_context()
+    address = _record_address(states, index)
+    drv = _driver.driver
+    if kind == _ONE_JUMP:
+        drv.nbh_xoro_one(address, kind, None, None)
+        return None
+    cell = ctx.take_result_cell()
+    try:
+        drv.nbh_xoro_one(address, kind, cell[0], None)
+        drv.nbh_stream_synchronize(None)
+        dtype = _ONE_RESULT[kind]
+        return cell[1][:dtype.itemsize].view(dtype)[0]
+    finally:
+        ctx.give_back_result_cell(cell)
 
 
 def init_xoroshiro128p_state(states, index, seed):
     """SplitMix64 step of `seed`; the same word goes into both halves."""
-    states = _host_states(states)
+    if _driver.is_device_memory(states):
+        devices.get_context()
+        _driver.driver.nbh_xoro_init_states(_record_address(states, index), 1, int(seed) & _M64, 0, None)
+        return
     z = (int(seed) + 0x9E3779B97F4A7C15) & _M64
     z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
     z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
@@ -137,7 +172,8 @@ def rotl(x, k):
 
 def xoroshiro128p_next(states, index):
     """Next uint64 of generator `index`; advances it."""
-    states = _host_states(states)
+    if _driver.is_device_memory(states):
+        return _on_device(states, index, _ONE_NEXT)
     index = int(index)
     s0 = int(states[index]["s0"])
     s1 = int(states[index]["s1"])
@@ -150,7 +186,8 @@ def xoroshiro128p_next(states, index):
 
 def xoroshiro128p_jump(states, index):
     """Advance generator `index` by 2**64 steps."""
-    states = _host_states(states)
+    if _driver.is_device_memory(states):
+        return _on_device(states, index, _ONE_JUMP)
     index = int(index)
     s0 = s1 = 0
     for word in (0xBEAC0467EBA5FACB, 0xD86B048B86AA9922):
@@ -172,10 +209,14 @@ def uint64_to_unit_float32(x):
 
 
 def xoroshiro128p_uniform_float32(states, index):
+    if _driver.is_device_memory(states):
+        return _on_device(states, index, _ONE_UNIFORM_F32)
     return uint64_to_unit_float32(xoroshiro128p_next(states, index))
 
 
 def xoroshiro128p_uniform_float64(states, index):
+    if _driver.is_device_memory(states):
+        return _on_device(states, index, _ONE_UNIFORM_F64)
     return uint64_to_unit_float64(xoroshiro128p_next(states, index))
 
 
@@ -185,6 +226,8 @@ TWO_PI_FLOAT64 = np.float64(2 * math.pi)
 
 def xoroshiro128p_normal_float32(states, index):
     """Box-Muller (cosine branch) in float32; uses two draws."""
+    if _driver.is_device_memory(states):
+        return _on_device(states, index, _ONE_NORMAL_F32)
     u1 = xoroshiro128p_uniform_float32(states, index)
     u2 = xoroshiro128p_uniform_float32(states, index)
     with np.errstate(divide="ignore"):
@@ -194,6 +237,8 @@ def xoroshiro128p_normal_float32(states, index):
 
 def xoroshiro128p_normal_float64(states, index):
     """Box-Muller (cosine branch); float32 uniforms and logarithm, float64 rest."""
+    if _driver.is_device_memory(states):
+        return _on_device(states, index, _ONE_NORMAL_F64)
     u1 = xoroshiro128p_uniform_float32(states, index)
     u2 = xoroshiro128p_uniform_float32(states, index)
     with np.errstate(divide="ignore"):

@@ -22,10 +22,16 @@ SUFFIX = {
     "u8": np.uint8, "u16": np.uint16, "u32": np.uint32, "u64": np.uint64,
     "f32": np.float32, "f64": np.float64,
 }
+# float16 (carried as its 16 bits in C) takes the four arithmetic operators; booleans
+# take add and mul here (their and / or / xor / max / min run as uint8)
+HALF_SUFFIX = {"f16": np.float16}
+BOOL_SUFFIX = {"b1": np.bool_}
+BOOL_OPS = ("add", "mul")
 # complex elements reduce with add and mul only
 COMPLEX_SUFFIX = {"c64": np.complex64, "c128": np.complex128}
 COMPLEX_OPS = ("add", "mul")
-_SUFFIX_OF = {np.dtype(v): k for k, v in list(SUFFIX.items()) + list(COMPLEX_SUFFIX.items())}
+_SUFFIX_OF = {np.dtype(v): k for k, v in list(SUFFIX.items()) + list(COMPLEX_SUFFIX.items())
+              + list(HALF_SUFFIX.items()) + list(BOOL_SUFFIX.items())}
 OPS = ("add", "mul", "max", "min")
 # bitwise functors exist for the integer element types only
 BITWISE_OPS = ("and", "or", "xor")
@@ -72,6 +78,15 @@ def lib():
             for sfx in COMPLEX_SUFFIX:
                 for fam in ("fold", "tree"):
                     getattr(L, f"orc_{fam}_{op}_{sfx}").argtypes = [_vp, _c_i64, _vp, _vp]
+        for fam in ("fold", "tree"):
+            for op in OPS:
+                getattr(L, f"orc_{fam}_{op}_f16").argtypes = [_vp, _c_i64, _vp, _vp]
+            for op in BOOL_OPS:
+                getattr(L, f"orc_{fam}_{op}_b1").argtypes = [_vp, _c_i64, _vp, _vp]
+        L.orc_f16_to_double.argtypes = [ctypes.c_uint16]
+        L.orc_f16_to_double.restype = ctypes.c_double
+        L.orc_f16_from_double.argtypes = [ctypes.c_double]
+        L.orc_f16_from_double.restype = ctypes.c_uint16
         L.orc_sum_exact_f32.argtypes = [_vp, _c_i64, _vp, _vp]
         L.orc_sum_exact_f64.argtypes = [_vp, _c_i64, _vp, _vp]
         L.orc_transpose.argtypes = [_vp, _vp] + [_c_i64] * 7
@@ -132,10 +147,19 @@ def fill(states, count, kind):
 # Reduction
 # ----------------------------------------------------------------------------
 
+def f16_to_double(bits):
+    return float(lib().orc_f16_to_double(int(bits)))
+
+
+def f16_from_double(x):
+    """Bit pattern of the float16 nearest to x (ties to even)."""
+    return int(lib().orc_f16_from_double(float(x)))
+
+
 def _reduce(fam, op, a, init):
     a = np.ascontiguousarray(a)
     sfx = _SUFFIX_OF[a.dtype]
-    ini = np.array([init]).astype(a.dtype)
+    ini = np.array([a.dtype.type(init)], dtype=a.dtype)     # arr.dtype.type(init), kernels/reduction.py:224
     out = np.zeros(1, a.dtype)
     getattr(lib(), f"orc_{fam}_{op}_{sfx}")(_ptr(a), a.size, _ptr(ini), _ptr(out))
     return out[0]

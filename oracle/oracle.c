@@ -13,6 +13,9 @@
  *       jump == next^(2^64) by GF(2) matrix power, big-int twin, closed forms)
  *   reduce tree order                     : pinned against a literal lock-step
  *       SIMT emulation (oracle/reduce_simt.py) and closed forms n(n+1)/2, n!
+ *   float16 arithmetic (software binary16): pinned against NumPy's float16 on every
+ *       bit pattern, and the float16 folds / trees against NumPy float16 folds and
+ *       the lock-step emulation run in float16
  *   transpose                             : pinned against numpy's a.T
  *   Box-Muller normals                    : parity unpinned at bit level.  The
  *       reference evaluates log/cos in NVIDIA libdevice, whose result bits no
@@ -350,6 +353,83 @@ DEFINE_REDUCE(add_c64, orc_c64, orc_c64, OP_ADD_C64)
 DEFINE_REDUCE(mul_c64, orc_c64, orc_c64, OP_MUL_C64)
 DEFINE_REDUCE(add_c128, orc_c128, orc_c128, OP_ADD_C128)
 DEFINE_REDUCE(mul_c128, orc_c128, orc_c128, OP_MUL_C128)
+
+/* float16 elements.  The reference's JIT lowers `a + b`, `a * b` on float16 operands to
+ * the GPU's native half-precision add / mul (one IEEE rounding to binary16 per
+ * operation) and max / min to comparisons of the two halves, so the accumulator is a
+ * half all the way (kernels/reduction.py:78-81: `tmp = reduce_op(tmp, arr[i])` keeps
+ * the element type).  Restated in software: a half is carried as its 16 bits; the sum
+ * and the product of two halves are exact in double (at most 40 and 22 significant
+ * bits), so one round-to-nearest-even from double to half is the one rounding.
+ *   parity of orc_f16_from_double / orc_f16_to_double: pinned against NumPy's float16
+ *   conversions on all 65536 bit patterns and on random doubles (tests/).  */
+typedef uint16_t orc_f16;
+
+double orc_f16_to_double(orc_f16 h)
+{
+    const int sign = h >> 15, e = (h >> 10) & 31, m = h & 1023;
+    double v;
+    if (e == 31)
+        v = m ? NAN : INFINITY;
+    else if (e == 0)
+        v = ldexp((double)m, -24);              /* subnormal: m * 2^-24 */
+    else
+        v = ldexp((double)(1024 + m), e - 25);  /* (1 + m/1024) * 2^(e-15) */
+    return sign ? -v : v;
+}
+
+orc_f16 orc_f16_from_double(double x)
+{
+    const orc_f16 sign = signbit(x) ? 0x8000u : 0u;
+    const double a = fabs(x);
+    if (isnan(x))
+        return (orc_f16)(sign | 0x7e00u);
+    if (a >= 65520.0)                           /* halfway between 65504 and 2^16 rounds to even: infinity */
+        return (orc_f16)(sign | 0x7c00u);
+    if (a < 0x1p-14) {
+        /* subnormal range: units of 2^-24; 1024 units is the smallest normal, whose
+         * bit pattern is exactly 1024 */
+        return (orc_f16)(sign | (orc_f16)nearbyint(ldexp(a, 24)));
+    }
+    int ex;
+    (void)frexp(a, &ex);                        /* a = f * 2^ex, f in [0.5, 1) */
+    int e = ex - 1;                             /* a in [2^e, 2^(e+1)) */
+    double r = nearbyint(ldexp(a, 10 - e));     /* in [1024, 2048], ties to even */
+    if (r == 2048.0) {
+        r = 1024.0;
+        e += 1;
+    }
+    return (orc_f16)(sign | (orc_f16)((e + 15) << 10) | (orc_f16)((int)r - 1024));
+}
+
+static inline orc_f16 f16_add(orc_f16 a, orc_f16 b)
+{
+    return orc_f16_from_double(orc_f16_to_double(a) + orc_f16_to_double(b));
+}
+static inline orc_f16 f16_mul(orc_f16 a, orc_f16 b)
+{
+    return orc_f16_from_double(orc_f16_to_double(a) * orc_f16_to_double(b));
+}
+#define OP_ADD_H(T, U, a, b) f16_add(a, b)
+#define OP_MUL_H(T, U, a, b) f16_mul(a, b)
+#define OP_MAX_H(T, U, a, b) ((orc_f16_to_double(b) > orc_f16_to_double(a)) ? (b) : (a))
+#define OP_MIN_H(T, U, a, b) ((orc_f16_to_double(b) < orc_f16_to_double(a)) ? (b) : (a))
+DEFINE_REDUCE(add_f16, orc_f16, orc_f16, OP_ADD_H)
+DEFINE_REDUCE(mul_f16, orc_f16, orc_f16, OP_MUL_H)
+DEFINE_REDUCE(max_f16, orc_f16, orc_f16, OP_MAX_H)
+DEFINE_REDUCE(min_f16, orc_f16, orc_f16, OP_MIN_H)
+
+/* Boolean elements under `a + b` and `a * b`.  The JIT types bool + bool and
+ * bool * bool as int64, and every store into the kernels' boolean arrays (shared
+ * partials :32-37, `partials[blkid]` :96, the result) converts back with `!= 0`; the
+ * per-thread accumulator of the strided loop (:78-81) is unified to int64 and holds a
+ * count (a product of 0/1 values) that cannot wrap.  Whatever the association, the
+ * result is therefore "any element or init is true" for +, "all are true" for *,
+ * as a boolean.  One byte per element, 0 or 1. */
+#define OP_ADD_B(T, U, a, b) ((T)((((int64_t)((a) != 0)) + ((int64_t)((b) != 0))) != 0))
+#define OP_MUL_B(T, U, a, b) ((T)((((int64_t)((a) != 0)) * ((int64_t)((b) != 0))) != 0))
+DEFINE_REDUCE(add_b1, uint8_t, uint8_t, OP_ADD_B)
+DEFINE_REDUCE(mul_b1, uint8_t, uint8_t, OP_MUL_B)
 
 /* Association-free yardsticks for the floating-point tolerance
  * |err| <= 2 n eps sum|x|: the sum and the sum of magnitudes accumulated in

@@ -240,3 +240,66 @@ def test_normals_over_every_float32_mantissa_of_u1():
             _say(kind, "binade", int(top).bit_length(), "worst ulp", u.max(), "mismatching", int((u > 0).sum()))
             assert u.max() <= 2.0
             np.testing.assert_array_equal(d.copy_to_host(), want_states)
+
+
+def test_scalar_functions_on_device_resident_states():
+    """numba_cuda/numba/cuda/random.py:96-238 called from host code on the array
+    create_xoroshiro128p_states returned: state and integer / uniform bits exact against
+    the oracle, normals within 2 ulp of it and bit-equal to the bulk fill."""
+    n = 6
+    states = cuda.random.create_xoroshiro128p_states(n, seed=1)
+    host = cref.init_states(n, 1)
+    np.testing.assert_array_equal(states.copy_to_host(), host)
+
+    # next: the raw 64-bit draws of generators 4 and -1, interleaved
+    twin = {4: np.array([host[4]["s0"], host[4]["s1"]], np.uint64),
+            5: np.array([host[5]["s0"], host[5]["s1"]], np.uint64)}
+    for i in range(20):
+        for idx, key in ((4, 4), (-1, 5)):
+            got = nrandom.xoroshiro128p_next(states, idx)
+            assert isinstance(got, np.uint64) and int(got) == cref.next_u64(twin[key]), (i, idx)
+    after = states.copy_to_host()
+    assert (after[4]["s0"], after[4]["s1"]) == tuple(twin[4])
+    assert (after[5]["s0"], after[5]["s1"]) == tuple(twin[5])
+    np.testing.assert_array_equal(after[:4], host[:4])            # the others did not move
+
+    # uniform draws: bit patterns of generator 0 (float32) and 1 (float64)
+    want32, st32 = cref.fill(host[0:1], 9, "uniform_f32")
+    got32 = np.array([nrandom.xoroshiro128p_uniform_float32(states, 0) for _ in range(9)])
+    assert got32.dtype == np.float32 and got32.tobytes() == want32.tobytes()
+    want64, st64 = cref.fill(host[1:2], 9, "uniform_f64")
+    got64 = np.array([nrandom.xoroshiro128p_uniform_float64(states, 1) for _ in range(9)])
+    assert got64.dtype == np.float64 and got64.tobytes() == want64.tobytes()
+    after = states.copy_to_host()
+    np.testing.assert_array_equal(after[0:1], st32)
+    np.testing.assert_array_equal(after[1:2], st64)
+
+    # normal draws of generators 2 and 3: two steps per value
+    for idx, kind, fn, dtype in ((2, "normal_f32", nrandom.xoroshiro128p_normal_float32, np.float32),
+                                 (3, "normal_f64", nrandom.xoroshiro128p_normal_float64, np.float64)):
+        want, st = cref.fill(host[idx:idx + 1], 11, kind)
+        bulk_states = cuda.to_device(host[idx:idx + 1])
+        bulk = cuda.device_array(11, dtype=dtype)
+        nrandom.xoroshiro128p_fill(bulk_states, bulk, 11, nrandom.NORMAL)
+        got = np.array([fn(states, idx) for _ in range(11)])
+        assert got.dtype == dtype
+        assert got.tobytes() == bulk.copy_to_host().tobytes()
+        assert _ulps(got, want).max() <= 2.0                       # tolerance: 2 ulp
+        np.testing.assert_array_equal(states.copy_to_host()[idx:idx + 1], st)
+
+    # jump: one step along the chain of subsequences
+    fresh = cuda.random.create_xoroshiro128p_states(4, seed=9)
+    chain = cref.init_states(5, 9)
+    for idx in range(4):
+        assert nrandom.xoroshiro128p_jump(fresh, idx) is None
+    np.testing.assert_array_equal(fresh.copy_to_host(), chain[1:])
+
+    # seeding one generator in place
+    nrandom.init_xoroshiro128p_state(fresh, 2, 12345)
+    s0, s1 = cref.seed_state(12345)
+    got = fresh.copy_to_host()
+    assert (int(got[2]["s0"]), int(got[2]["s1"])) == (s0, s1)
+    np.testing.assert_array_equal(got[[0, 1, 3]], chain[[1, 2, 4]])
+
+    with pytest.raises(IndexError):
+        nrandom.xoroshiro128p_next(states, n)

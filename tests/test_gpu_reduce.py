@@ -162,8 +162,73 @@ def test_boolean_arrays_any_all_parity():
     res = cuda.device_array(1, np.bool_)
     any_(d[::2], res=res)
     assert res.copy_to_host()[0] == a[::2].any()
-    with pytest.raises(NotImplementedError, match="booleans"):
-        cuda.Reduce(lambda a, b: a + b)(a)
+
+
+def test_boolean_sums_and_products():
+    """`a + b` / `a * b` on booleans: int64 in the reference's JIT, converted back with
+    `!= 0` at every store into its boolean arrays - any / all, as np.bool_."""
+    rng = np.random.default_rng(9)
+    add, mul = cuda.Reduce(lambda a, b: a + b), cuda.Reduce(lambda a, b: a * b)
+    for n in (1, 2, 63, 65, 5000, 300001, 2**24 + 5):
+        for p in (0.0, 1.0, 0.5, 1.0 / n, 1.0 - 1.0 / n):
+            a = rng.random(n) < p
+            _say("bool add/mul", n, p)
+            d = cuda.to_device(a)
+            for init in (0, 1, 2, False, True):
+                got_add, got_mul = add(d, init=init), mul(d, init=init)
+                assert got_add.dtype == np.bool_ and got_mul.dtype == np.bool_
+                assert got_add == cref.tree("add", a, init) == cref.fold("add", a, init) == (a.any() or bool(init))
+                assert got_mul == cref.tree("mul", a, init) == cref.fold("mul", a, init) == (a.all() and bool(init))
+    res = cuda.device_array(1, np.bool_)
+    add(d[::2], res=res)
+    assert res.copy_to_host()[0] == a[::2].any()
+
+
+def test_float16_reductions():
+    """float16 is accumulated in float16 (one rounding per operation), like the reference's
+    JIT does.  Bar: max / min bit-exact; sums bit-exact where every partial sum is a
+    float16 in any association; other sums within 2 n eps sum|x| (eps = 2^-11) of the exact
+    sum and of the reference-order value; products within 4 n eps relative."""
+    rng = np.random.default_rng(10)
+    add, mul = cuda.Reduce(lambda a, b: a + b), cuda.Reduce(lambda a, b: a * b)
+    mx, mn = cuda.Reduce(lambda a, b: max(a, b)), cuda.Reduce(lambda a, b: min(a, b))
+    eps = 2.0 ** -11
+    for n in (1, 2, 7, 8, 9, 63, 64, 65, 511, 512, 513, 4097, 100003, 2**22 + 3):
+        _say("float16 reduce", n)
+        a = (rng.standard_normal(n) * 8).astype(np.float16)
+        d = cuda.to_device(a)
+        got = [mx(d, init=-np.inf), mn(d, init=np.inf)]
+        assert all(g.dtype == np.float16 for g in got)
+        assert got[0].tobytes() == cref.tree("max", a, -np.inf).tobytes() == a.max().tobytes()
+        assert got[1].tobytes() == cref.tree("min", a, np.inf).tobytes() == a.min().tobytes()
+        # small integers whose running totals stay below 2048 in magnitude: exact in every order
+        k = rng.integers(-3, 4, n).astype(np.float16)
+        if np.abs(k.astype(np.float64)).sum() < 2048:
+            got = add(k, init=5)
+            assert got.dtype == np.float16
+            assert got.tobytes() == cref.tree("add", k, 5).tobytes() == cref.fold("add", k, 5).tobytes()
+            assert float(got) == k.astype(np.float64).sum() + 5
+        if n <= 4097:
+            got = float(add(d, init=0))
+            exact = a.astype(np.float64).sum()
+            bound = 2 * n * eps * np.abs(a.astype(np.float64)).sum() + eps * abs(exact)    # tolerance
+            assert abs(got - exact) <= bound, (n, got, exact)
+            assert abs(got - float(cref.tree("add", a, 0))) <= 2 * bound
+            b = (1.0 + rng.standard_normal(n) * 2e-3).astype(np.float16)
+            got = float(mul(b, init=1))
+            exact = float(np.prod(b.astype(np.float64)))
+            assert abs(got - exact) <= (4 * n + 1) * eps * abs(exact), (n, got, exact)     # tolerance
+    # the accumulator is a half: 2^20 ones overflow it (65504 is the largest float16),
+    # in the reference's association as in this one
+    ones = np.ones(2**20, np.float16)
+    assert float(add(ones)) == float(cref.tree("add", ones, 0)) == np.inf
+    # strided view, device result slot, offset views
+    d = cuda.to_device(a)
+    res = cuda.device_array(1, np.float16)
+    mx(d[::3], res=res, init=-np.inf)
+    assert res.copy_to_host()[0] == a[::3].max()
+    for lo in (1, 2, 3, 7, 9):
+        assert mn(d[lo:], init=np.inf) == a[lo:].min()
 
 
 @pytest.mark.parametrize("dtype", [np.complex64, np.complex128])

@@ -262,3 +262,64 @@ def test_extents_against_numpy(shape, strides, itemsize):
     idx = np.indices(shape).reshape(len(shape), -1).T if shape else np.zeros((1, 0), int)
     offs = (idx * np.asarray(strides, int)).sum(axis=1) if shape else np.array([0])
     assert lo == offs.min() and hi == offs.max() + itemsize
+
+
+# ---------------------------------------------------------------- float16 and boolean elements
+
+def test_software_float16_matches_numpy_on_every_bit_pattern():
+    bits = np.arange(65536, dtype=np.uint16)
+    as_double = bits.view(np.float16).astype(np.float64)
+    for b, want in zip(bits.tolist(), as_double.tolist()):
+        got = cref.f16_to_double(b)
+        assert got == want or (got != got and want != want), b
+        if want == want:
+            assert cref.f16_from_double(want) == b, b
+    # rounding: random doubles, the overflow boundary, the subnormal range, ties
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(30000) * 10.0 ** rng.integers(-9, 6, 30000),
+                        [65519.999, 65520.0, 65504.0, 1e-8, 2.9802322387695312e-08, 2.98e-8, 8.9406967163085938e-08,
+                         1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 2.0 ** -14 - 2.0 ** -25, -0.0]])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    got = np.array([cref.f16_from_double(v) for v in x], dtype=np.uint16)
+    assert (want == got).all()
+
+
+@pytest.mark.parametrize("n", [1, 2, 31, 33, 127, 128, 129, 1000, 4097, 8192, 8321, 20000])
+def test_float16_folds_and_trees_round_once_per_operation(n):
+    """Left fold against functools.reduce over NumPy float16 scalars (NumPy computes
+    each operation in float32 and rounds to float16: one effective rounding), tree
+    against the statement-by-statement kernel emulation run on float16 arrays."""
+    import functools
+    rng = np.random.default_rng(n)
+    a = (rng.standard_normal(n) * 4).astype(np.float16)
+    init = np.float16(0.37)
+    with np.errstate(over="ignore"):
+        for op, fn in (("add", lambda x, y: x + y), ("max", lambda x, y: y if y > x else x),
+                       ("min", lambda x, y: y if y < x else x)):
+            assert cref.fold(op, a, init).tobytes() == functools.reduce(fn, a, init).tobytes(), (op, n)
+            assert cref.tree(op, a, init).tobytes() == reduce_simt.reduce(op, a, init).tobytes(), (op, n)
+        b = (1.0 + rng.standard_normal(n) * 1e-2).astype(np.float16)
+        assert cref.fold("mul", b, 1).tobytes() == functools.reduce(lambda x, y: x * y, b, np.float16(1)).tobytes()
+        assert cref.tree("mul", b, 1).tobytes() == reduce_simt.reduce("mul", b, 1).tobytes()
+    assert cref.fold("add", a, init).dtype == np.float16
+
+
+def test_float16_sum_shows_its_own_rounding():
+    # 2048 + 1 is not a float16: a half accumulator sticks at 2048, a wider one would not
+    a = np.ones(4000, np.float16)
+    assert cref.fold("add", a, 0) == 2048
+    assert cref.tree("add", a, 0) == 4000        # 8192 lanes hold one element each; the tree adds equal powers of two
+
+
+@pytest.mark.parametrize("n", [1, 2, 33, 127, 129, 5000, 8321])
+def test_boolean_sums_and_products_are_any_and_all(n):
+    rng = np.random.default_rng(n)
+    for p in (0.0, 1.0, 0.5, 1.0 / n):
+        a = rng.random(n) < p
+        for init in (False, True, 0, 1, 2):
+            for fam in (cref.fold, cref.tree):
+                got = fam("add", a, init)
+                assert got.dtype == np.bool_ and got == (a.any() or bool(init)), (n, p, init)
+                got = fam("mul", a, init)
+                assert got.dtype == np.bool_ and got == (a.all() and bool(init)), (n, p, init)

@@ -81,11 +81,13 @@ def test_reduce_host_side_contract(fake_gpu):
     assert red(cuda.device_array(10, np.int16), size=0, init=2) == 2
     assert not [c for c in fake_gpu.calls if c[0] in ("h2d", "d2h")]
     with pytest.raises(NotImplementedError, match="dtype"):
-        red(np.zeros(4, np.float16))
+        red(np.zeros(4, np.dtype("S4")))
     with pytest.raises(TypeError, match="not defined for complex64"):
         cuda.reduce(lambda a, b: max(a, b))(np.zeros(4, np.complex64))
-    with pytest.raises(NotImplementedError, match="does not add or multiply booleans"):
-        red(np.zeros(4, np.bool_))
+    # booleans under + run as the uint8 `or` kernel, float16 has kernels of its own
+    assert red._codes_for(np.dtype(np.bool_)) == (5, 4)
+    assert cuda.reduce(lambda a, b: a * b)._codes_for(np.dtype(np.bool_)) == (4, 4)
+    assert red._codes_for(np.dtype(np.float16)) == (0, 12)
     with pytest.raises(TypeError, match="bitwise xor is not defined for float32"):
         cuda.reduce(lambda a, b: a ^ b)(np.zeros(4, np.float32))
 
@@ -121,11 +123,31 @@ def test_random_host_scalar_functions_match_the_oracle():
         assert abs(nrandom.xoroshiro128p_normal_float64(b, t) - n64[t]) <= 4 * np.spacing(abs(n64[t]))
 
 
-def test_device_states_are_refused_by_scalar_functions(fake_gpu):
+def test_scalar_functions_on_device_states_go_through_the_one_generator_kernel(fake_gpu):
+    """Host logic only (there is no kernel on the fake library): which record address,
+    which kind and which output cell the per-generator functions pass on."""
     from numba_cuda_amd import random as nrandom
     d = cuda.device_array(4, dtype=nrandom.xoroshiro128p_dtype)
-    with pytest.raises(TypeError, match="xoroshiro128p_fill"):
-        nrandom.xoroshiro128p_uniform_float32(d, 0)
+    base = d.device_ctypes_pointer.value
+    calls = []
+
+    def nbh_xoro_one(state, kind, out, stream):
+        calls.append((state, kind, out))
+        if out:
+            ctypes.c_uint64.from_address(out).value = 0x3FF8000000000000       # 1.5 as a double
+        return 0
+
+    import ctypes
+    fake_gpu.nbh_xoro_one = nbh_xoro_one
+    got = nrandom.xoroshiro128p_uniform_float64(d, 2)
+    assert isinstance(got, np.float64) and got == 1.5
+    assert calls[-1][:2] == (base + 32, 3) and calls[-1][2]
+    got = nrandom.xoroshiro128p_next(d, -1)
+    assert isinstance(got, np.uint64) and calls[-1][:2] == (base + 48, 0)
+    assert nrandom.xoroshiro128p_jump(d, 0) is None and calls[-1] == (base, 1, None)
+    assert isinstance(nrandom.xoroshiro128p_normal_float32(d, 1), np.float32) and calls[-1][1] == 4
+    with pytest.raises(IndexError):
+        nrandom.xoroshiro128p_uniform_float32(d, 4)
     with pytest.raises(TypeError, match="device array"):
         nrandom.xoroshiro128p_fill(np.zeros(4, nrandom.xoroshiro128p_dtype), d)
 
