@@ -241,9 +241,40 @@ def _workload(name, cuda):
             for s in streams[1:]:
                 s.synchronize()
 
+        def extras():
+            """Where a call's time goes: the issuing loop alone (no waiting), and the same
+            4096 launches of this kernel issued through the bare native call with precomputed
+            integer arguments - what the runtime's launch path costs per call, the floor
+            under any per-call interface."""
+            from numba_cuda_amd.cudadrv import driver as drv
+            from numba_cuda_amd.kernels import reduction
+            cuda.synchronize()
+            t0 = time.perf_counter()
+            for r in range(rows):
+                add(views[r], res=slots[r], stream=streams[r & 3])
+            issue = time.perf_counter() - t0
+            cuda.synchronize()
+            lib, ctx = drv.driver.lib, cuda.current_context()
+            entry = lib._reduce_entry
+            scratch = [ctx.reduce_scratch(s.handle) for s in streams]
+            handles = [s.handle for s in streams]
+            init_ptr = reduction._init_buffer(np.dtype(np.float32), 0)
+            a, o = dm.gpu_data.device_pointer, out.gpu_data.device_pointer
+            args = [(entry, 0, 8, a + r * cols * 4, cols, 4, init_ptr, o + 4 * r, scratch[r & 3][0], scratch[r & 3][1],
+                     handles[r & 3]) for r in range(rows)]
+            call = drv._hostbuf.call_reduce
+            t0 = time.perf_counter()
+            for t in args:
+                call(*t)
+            floor = time.perf_counter() - t0
+            cuda.synchronize()
+            return {"issue_us_per_call": round(issue / rows * 1e6, 3),
+                    "native_launch_us_per_call": round(floor / rows * 1e6, 3)}
+
         return dict(desc="4096 x (65536 fp32) row sums round-robin over 4 streams, seed 3", dtype="f32",
                     algo_bytes=host.nbytes, units=rows, step=step, stream=streams[0], host=host,
-                    kernel="reduce_kernel", keep=(dm, out, streams, views, slots), calls_per_step=rows)
+                    kernel="reduce_kernel", keep=(dm, out, streams, views, slots), calls_per_step=rows,
+                    extras=extras)
     raise SystemExit("unknown workload %s" % name)
 
 
@@ -319,6 +350,8 @@ def measure(cuda, name, steps, warmup, cpu_seconds):
            "roofline": roofline, "cpu_baseline": cpu}
     if "calls_per_step" in w:
         out["us_per_call"] = round(ms_per_step * 1e3 / w["calls_per_step"], 3)
+    if "extras" in w:
+        out.update(w["extras"]())
     return out
 
 

@@ -10,12 +10,17 @@
  *   extents(obj)            half-open byte range [lo, hi) its items occupy, strides of
  *                           either sign, empty when any extent is zero
  *   extents_of(shape, strides, itemsize)  the same from a description, relative to 0
+ *   call_reduce(entry, op, dtype, in, n, stride, init, out, scratch, scratch_bytes, stream)
+ *                           calls the library's nbh_reduce through its address, all
+ *                           arguments plain integers: the launch path of Reduce.__call__
+ *                           without the per-argument conversions of a ctypes call
  *
  * Counterpart of numba_cuda/numba/cuda/cext/mviewbuf.c:48-70 (address), :76-135 and
  * :138-209 (extents), :212-363 (the buffer-exporting type).
  */
 #define PY_SSIZE_T_CLEAN
 #include <Python.h>
+#include <stdint.h>
 
 /* ---- byte range of a strided block ------------------------------------------------ */
 
@@ -164,7 +169,56 @@ static PyObject *hb_extents_of(PyObject *mod, PyObject *args)
     return Py_BuildValue("nn", lo, hi);
 }
 
+/* ---- the reduction launch, called thousands of times a second ------------------------ */
+
+typedef int (*nbh_reduce_fn)(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init,
+                             void *out, void *scratch, size_t scratch_bytes, void *stream);
+
+static int as_word(PyObject *o, unsigned long long *out)
+{
+    /* addresses and sizes arrive as non-negative Python ints, None stands for 0 */
+    if (o == Py_None) {
+        *out = 0;
+        return 0;
+    }
+    unsigned long long v = PyLong_AsUnsignedLongLong(o);
+    if (v == (unsigned long long)-1 && PyErr_Occurred())
+        return -1;
+    *out = v;
+    return 0;
+}
+
+static PyObject *hb_call_reduce(PyObject *mod, PyObject *const *args, Py_ssize_t nargs)
+{
+    if (nargs != 11) {
+        PyErr_SetString(PyExc_TypeError, "call_reduce takes 11 arguments");
+        return NULL;
+    }
+    unsigned long long entry, in, init, out, scratch, scratch_bytes, stream;
+    if (as_word(args[0], &entry) || as_word(args[3], &in) || as_word(args[6], &init) || as_word(args[7], &out) ||
+        as_word(args[8], &scratch) || as_word(args[9], &scratch_bytes) || as_word(args[10], &stream))
+        return NULL;
+    const long op = PyLong_AsLong(args[1]), dtype = PyLong_AsLong(args[2]);
+    const long long n = PyLong_AsLongLong(args[4]), stride = PyLong_AsLongLong(args[5]);
+    if (PyErr_Occurred())
+        return NULL;
+    if (!entry) {
+        PyErr_SetString(PyExc_ValueError, "call_reduce: null entry point");
+        return NULL;
+    }
+    int status;
+    Py_BEGIN_ALLOW_THREADS
+    status = ((nbh_reduce_fn)(uintptr_t)entry)((int)op, (int)dtype, (const void *)(uintptr_t)in, (int64_t)n,
+                                               (int64_t)stride, (const void *)(uintptr_t)init,
+                                               (void *)(uintptr_t)out, (void *)(uintptr_t)scratch,
+                                               (size_t)scratch_bytes, (void *)(uintptr_t)stream);
+    Py_END_ALLOW_THREADS
+    return PyLong_FromLong(status);
+}
+
 static PyMethodDef hb_methods[] = {
+    {"call_reduce", (PyCFunction)(void (*)(void))hb_call_reduce, METH_FASTCALL,
+     "call_reduce(entry, op, dtype, in, n, stride, init, out, scratch, scratch_bytes, stream) -> status"},
     {"address", hb_address, METH_VARARGS, "address(obj, writable=True) -> int"},
     {"extents", hb_extents, METH_O, "extents(obj) -> (lo, hi)"},
     {"extents_of", hb_extents_of, METH_VARARGS, "extents_of(shape, strides, itemsize) -> (lo, hi)"},

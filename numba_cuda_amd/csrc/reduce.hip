@@ -386,6 +386,13 @@ int launch(const void *in, int64_t n, int64_t stride, const void *init, void *ou
 
     const int64_t per_block = (int64_t)kBlock * kUnroll;
     int64_t grid = (units + per_block - 1) / per_block;
+    // Small inputs are latency, not bandwidth: spread them over up to 32 workgroups with
+    // one load per lane (256 KiB: 4.1 -> 3.8 us, against 2.4 - 2.7 us for an empty kernel).
+    if (grid < 32) {
+        grid = (units + kBlock - 1) / kBlock;
+        if (grid > 32)
+            grid = 32;
+    }
     int64_t cap = (int64_t)nbh_cu_count() * kGridPerCU;
     constexpr int64_t kSlots = (int64_t)kMaxGrid * 8 / (sizeof(T) > 8 ? 16 : 8);  // partials that fit the scratch
     if (cap > kSlots)

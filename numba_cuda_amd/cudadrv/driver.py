@@ -1155,8 +1155,9 @@ class OwnedPointer:
             raise AssertionError("a view into owned memory cannot have a finalizer of its own")
         self._mem = memptr
         self._view = memptr if view is None else view
-        # read for every kernel argument: worth a real attribute
+        # read for every kernel argument: worth real attributes
         self.device_ctypes_pointer = self._view.device_ctypes_pointer
+        self.device_pointer = self._view.device_pointer
         memptr.refct += 1
         weakref.finalize(self, _let_go, memptr)
 

@@ -219,36 +219,60 @@ class Reduce:
         stream : stream to work on (0: the default stream)
         Returns the result as a NumPy scalar, or None when `res` is given.
         """
+        # This is the whole per-call cost of small reductions (a 256 KiB row takes the
+        # device 3 us): plain attribute reads, dictionary look-ups and one native call.
         if arr.ndim != 1:
             raise TypeError("only support 1D array")
         if size is not None:
             arr = arr[:size]
         dtype = arr.dtype
-        if arr.size < 1:
+        n = arr.size
+        if n < 1:
             return dtype.type(init)          # `res` is left untouched, as in the reference
 
         codes = self._codes.get(dtype)
         if codes is None:
             codes = self._codes[dtype] = self._codes_for(dtype)
-        opcode, code = codes
 
-        ctx = devices.get_context()
-        if not _driver.is_device_memory(arr):
-            # host input: implicit transfer, as a kernel argument would get
-            arr, _ = devicearray.auto_device(arr, stream=stream)
+        ctx = getattr(_thread_state, "ctx", None)       # devices.get_context() without the calls
+        if ctx is None or not ctx.prepared:
+            ctx = devices.get_context()
+        try:
+            in_ptr = arr.gpu_data.device_pointer
+        except AttributeError:
+            if not _driver.is_device_memory(arr):
+                # host input: implicit transfer, as a kernel argument would get
+                arr, _ = devicearray.auto_device(arr, stream=stream)
+            in_ptr = arr.device_ctypes_pointer.value
 
-        hstream = stream.handle if type(stream) is _driver.Stream else _driver._stream_handle(stream)
-        scratch_ptr, scratch_bytes = ctx.reduce_scratch(hstream)
-        init_ptr = _init_buffer(dtype, init)
-        drv = _driver.driver
+        hstream = stream.handle if stream.__class__ is _Stream else _driver._stream_handle(stream)
+        scratch = ctx._scratch.get(hstream)
+        if scratch is None or hstream == _PER_THREAD:
+            scratch = ctx.reduce_scratch(hstream)
+        init_ptr = _INT_INIT.get((dtype, init)) if init.__class__ is int else None
+        if init_ptr is None:
+            init_ptr = _init_buffer(dtype, init)
+        lib = _driver.driver.lib
+        try:
+            entry = lib._reduce_entry
+        except AttributeError:
+            entry = lib._reduce_entry = _entry_address(lib)
+
         if res is not None:
             if res.dtype != dtype:
                 raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
-            rc = drv.lib.nbh_reduce(opcode, code, arr.device_ctypes_pointer.value, arr.size,
-                                    arr.strides[0], init_ptr, res.device_ctypes_pointer.value,
-                                    scratch_ptr, scratch_bytes, hstream or None)
+            try:
+                out_ptr = res.gpu_data.device_pointer
+            except AttributeError:
+                out_ptr = res.device_ctypes_pointer.value
+            if entry:
+                rc = _call_reduce(entry, codes[0], codes[1], in_ptr, n, arr.strides[0], init_ptr, out_ptr,
+                                  scratch[0], scratch[1], hstream)
+            else:
+                rc = lib.nbh_reduce(codes[0], codes[1], in_ptr, n, arr.strides[0], init_ptr, out_ptr,
+                                    scratch[0], scratch[1], hstream or None)
             if rc:
-                drv.check("nbh_reduce", rc)
+                _driver.driver.check("nbh_reduce", rc)
             return None
         # The value is wanted on the host: the kernel writes it into a cell of host
         # memory the device can address (taken for this call alone, so that calls from
@@ -256,15 +280,29 @@ class Reduce:
         # stream and reads the cell - no copy back.
         cell = ctx.take_result_cell()
         try:
-            rc = drv.lib.nbh_reduce(opcode, code, arr.device_ctypes_pointer.value, arr.size,
-                                    arr.strides[0], init_ptr, cell[0],
-                                    scratch_ptr, scratch_bytes, hstream or None)
+            rc = lib.nbh_reduce(codes[0], codes[1], in_ptr, n, arr.strides[0], init_ptr, cell[0],
+                                scratch[0], scratch[1], hstream or None)
             if rc:
-                drv.check("nbh_reduce", rc)
-            drv.nbh_stream_synchronize(hstream or None)
+                _driver.driver.check("nbh_reduce", rc)
+            _driver.driver.nbh_stream_synchronize(hstream or None)
             return cell[1][:dtype.itemsize].view(dtype)[0]
         finally:
             ctx.give_back_result_cell(cell)
+
+
+_Stream = _driver.Stream
+_PER_THREAD = _driver.HIP_STREAM_PER_THREAD
+_thread_state = devices._runtime._tls
+_call_reduce = _driver._hostbuf.call_reduce
+
+def _entry_address(lib):
+    """Address of the library's nbh_reduce for call_reduce, kept on the library object
+    (0: not a native function, e.g. a test double - call it the ordinary way)."""
+    import ctypes
+    try:
+        return ctypes.cast(lib.nbh_reduce, ctypes.c_void_p).value or 0
+    except (TypeError, ctypes.ArgumentError, AttributeError):
+        return 0
 
 
 _DTYPE_CODE = {np.dtype(name): code for name, code in _lib.DTYPE_CODES.items()}
@@ -275,6 +313,10 @@ _BOOL = np.dtype(np.bool_)
 _INIT_CACHE = {}
 
 
+# (dtype, int value) -> address: the common case (`init=0`) without building an array first
+_INT_INIT = {}
+
+
 def _init_buffer(dtype, init):
     """Address of a host copy of `init` converted to `dtype`.  The copies are kept for
     the life of the process, found again by the bit pattern of the converted value
@@ -282,15 +324,17 @@ def _init_buffer(dtype, init):
     buf = np.array([dtype.type(init)], dtype=dtype)
     key = (dtype, buf.tobytes())
     kept = _INIT_CACHE.get(key)
-    if kept is not None:
-        return kept[1]
-    if len(_INIT_CACHE) < 4096:
-        _INIT_CACHE[key] = (buf, buf.ctypes.data)
-        return buf.ctypes.data
-    _KEEPALIVE.append(buf)
-    if len(_KEEPALIVE) > 64:
-        del _KEEPALIVE[:32]
-    return buf.ctypes.data
+    if kept is None:
+        if len(_INIT_CACHE) < 4096:
+            kept = _INIT_CACHE[key] = (buf, buf.ctypes.data)
+        else:
+            _KEEPALIVE.append(buf)
+            if len(_KEEPALIVE) > 64:
+                del _KEEPALIVE[:32]
+            return buf.ctypes.data
+    if init.__class__ is int and len(_INT_INIT) < 4096:
+        _INT_INIT[dtype, init] = kept[1]
+    return kept[1]
 
 
 _KEEPALIVE = []

@@ -323,6 +323,33 @@ def test_stream_and_result_slot_round_robin():
     assert v.tobytes() == got[5].tobytes()
 
 
+def test_batched_row_sums_full_shape_4096_rows_over_four_streams():
+    """The batched configuration at its real shape: 4096 independent float32 sums over the
+    65 536-item rows of a uniform [-1, 1) matrix (seed 3), each issued with its own call into a
+    slot of one device vector, round-robin over 4 streams.  Every row against the exact sum
+    (tolerance 2 n eps sum|x|) and, bit for bit, against the same reduction issued alone."""
+    rng = np.random.default_rng(3)
+    rows, cols = 4096, 65536
+    m = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
+    dm = cuda.to_device(m)
+    out = cuda.device_array(rows, dtype=np.float32)
+    streams = [cuda.stream() for _ in range(4)]
+    views = [dm[i] for i in range(rows)]
+    slots = [out[i:i + 1] for i in range(rows)]
+    _say("batched: issuing", rows, "reductions")
+    for i in range(rows):
+        sum_reduce(views[i], res=slots[i], stream=streams[i & 3])
+    for s in streams:
+        s.synchronize()
+    got = out.copy_to_host()
+    eps = np.finfo(np.float32).eps
+    for i in range(rows):
+        exact, sum_abs = cref.sum_exact(m[i])
+        assert abs(float(got[i]) - exact) <= 2 * cols * eps * sum_abs, i      # tolerance
+    for i in (0, 1, 2, 3, 1000, 4095):
+        assert sum_reduce(views[i]).tobytes() == got[i].tobytes()
+
+
 # ---- full HBM-scale inputs, seed 1 ---------------- --------------------------------
 
 def test_fullsize_float32_sum_and_max_2_pow_28():
