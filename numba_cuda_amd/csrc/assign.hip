@@ -301,7 +301,7 @@ int launch_fill_strided(void *dst, const Dims &d, int64_t itemsize, int64_t item
 
 int nbh_flat_copy(void *dst, const void *src, int64_t nbytes, hipStream_t stream)
 {
-    nbh_pool_note_stream(stream);
+    nbh_stream_report report(stream);
     const uint64_t mix = (uint64_t)(uintptr_t)dst | (uint64_t)(uintptr_t)src | (uint64_t)nbytes | 16u;
     switch (low_bit(mix)) {
     case 1: return launch_flat<1>(dst, src, nbytes, stream);
@@ -352,7 +352,7 @@ extern "C" int nbh_fill(void *dst, int ndim, const int64_t *shape, const int64_t
         mix |= (uint64_t)d.dst_stride[k];
     const int64_t g = low_bit(mix);
     hipStream_t s = nbh_hip_stream(stream);
-    nbh_pool_note_stream(s);
+    nbh_stream_report report(s);
     const unsigned char *item = static_cast<const unsigned char *>(value);
     const bool flat = d.nd == 0 || (d.nd == 1 && d.dst_stride[0] == itemsize);
     if (flat) {
@@ -418,7 +418,7 @@ extern "C" int nbh_assign(void *dst, const void *src, int ndim, const int64_t *s
         mix |= (uint64_t)d.dst_stride[k] | (uint64_t)d.src_stride[k];
     const int64_t g = low_bit(mix);
     hipStream_t s = nbh_hip_stream(stream);
-    nbh_pool_note_stream(s);
+    nbh_stream_report report(s);
 
     const bool flat = d.nd == 0 || (d.nd == 1 && d.dst_stride[0] == itemsize && d.src_stride[0] == itemsize);
     if (flat) {

@@ -23,9 +23,19 @@ static inline hipStream_t nbh_hip_stream(nbh_stream_t s) { return (hipStream_t)s
 int nbh_cu_count();
 
 // The caching pool (pool.hip) must know which streams have had work submitted: every
-// entry point that takes a stream reports it here (a no-op until the pool is in use).
+// entry point that takes a stream reports it (a no-op until the pool is in use).
 void nbh_pool_note_stream(hipStream_t stream);
 void nbh_pool_forget_stream(hipStream_t stream);
+// The report has to come AFTER the work is in the stream's queue (a block freed by
+// another thread in between must not be covered by an event recorded too early):
+// declare one of these at the top of an entry point and it reports on the way out.
+struct nbh_stream_report {
+    hipStream_t stream;
+    explicit nbh_stream_report(hipStream_t s) : stream(s) {}
+    ~nbh_stream_report() { nbh_pool_note_stream(stream); }
+    nbh_stream_report(const nbh_stream_report &) = delete;
+    nbh_stream_report &operator=(const nbh_stream_report &) = delete;
+};
 
 // Large copies between pageable host memory and the device through a
 // ring of page-locked buffers and a few copy threads (hostcopy.hip).  0: done;

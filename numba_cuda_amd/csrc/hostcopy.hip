@@ -28,6 +28,8 @@
 #include <thread>
 #include <vector>
 
+#include <unistd.h>
+
 namespace {
 
 constexpr size_t kChunkMax = (size_t)16 << 20;  // bytes per staging buffer
@@ -130,9 +132,18 @@ struct Pipeline {
     int helpers = -1;     // -1: not read from the environment yet
 };
 
+// Never destroyed: no thread joins at exit.  A forked child inherits the object but
+// neither the helper threads nor a usable lock (another thread may have held it): it
+// starts over with a pipeline of its own.
 Pipeline &pipeline()
 {
-    static Pipeline *p = new Pipeline;  // never destroyed: no thread joins at exit
+    static Pipeline *p = nullptr;
+    static pid_t owner = 0;
+    const pid_t me = getpid();
+    if (!p || owner != me) {
+        p = new Pipeline;
+        owner = me;
+    }
     return *p;
 }
 
@@ -156,9 +167,12 @@ int prepare(Pipeline &p, Ring **out)
         return -1;
     Ring &r = p.rings[dev];
     if (!r.ready) {
+        // what an earlier, failed attempt already made is kept and not made again
         for (int k = 0; k < kRing; ++k) {
-            NBH_TRY(hipHostMalloc((void **)&r.buf[k], kChunkMax, hipHostMallocDefault));
-            NBH_TRY(hipEventCreateWithFlags(&r.landed[k], hipEventDisableTiming));
+            if (!r.buf[k])
+                NBH_TRY(hipHostMalloc((void **)&r.buf[k], kChunkMax, hipHostMallocDefault));
+            if (!r.landed[k])
+                NBH_TRY(hipEventCreateWithFlags(&r.landed[k], hipEventDisableTiming));
         }
         r.ready = true;
     }
@@ -206,17 +220,24 @@ int nbh_staged_d2h(void *dst, const void *src, size_t nbytes, hipStream_t stream
         NBH_TRY(hipEventRecord(ring->landed[k], stream));
         return 0;
     };
-    for (size_t i = 0; i < std::min<size_t>(kRing, chunks); ++i)
-        if ((rc = fetch(i)))
-            return rc;
-    for (size_t i = 0; i < chunks; ++i) {
-        const int k = (int)(i % kRing);
-        NBH_TRY(hipEventSynchronize(ring->landed[k]));
-        p.crew->copy((char *)dst + i * kChunk, ring->buf[k], span(i));
-        if (i + kRing < chunks && (rc = fetch(i + kRing)))  // the buffer is free again
-            return rc;
-    }
-    return 0;
+    auto run = [&]() -> int {
+        for (size_t i = 0; i < std::min<size_t>(kRing, chunks); ++i)
+            if (int e = fetch(i))
+                return e;
+        for (size_t i = 0; i < chunks; ++i) {
+            const int k = (int)(i % kRing);
+            NBH_TRY(hipEventSynchronize(ring->landed[k]));
+            p.crew->copy((char *)dst + i * kChunk, ring->buf[k], span(i));
+            if (i + kRing < chunks)  // the buffer is free again
+                if (int e = fetch(i + kRing))
+                    return e;
+        }
+        return 0;
+    };
+    rc = run();
+    if (rc)  // chunks already issued still write into the ring: nobody may use it before they are done
+        (void)hipStreamSynchronize(stream);
+    return rc;
 }
 
 int nbh_staged_h2d(void *dst, const void *src, size_t nbytes, hipStream_t stream)
@@ -233,14 +254,20 @@ int nbh_staged_h2d(void *dst, const void *src, size_t nbytes, hipStream_t stream
         return -1;
     }
     const size_t chunks = (nbytes + kChunk - 1) / kChunk;
-    for (size_t i = 0; i < chunks; ++i) {
-        const int k = (int)(i % kRing);
-        const size_t n = std::min(kChunk, nbytes - i * kChunk);
-        if (i >= (size_t)kRing)  // the DMA that read this buffer kRing chunks ago must be over
-            NBH_TRY(hipEventSynchronize(ring->landed[k]));
-        p.crew->copy(ring->buf[k], (const char *)src + i * kChunk, n);
-        NBH_TRY(hipMemcpyAsync((char *)dst + i * kChunk, ring->buf[k], n, hipMemcpyHostToDevice, stream));
-        NBH_TRY(hipEventRecord(ring->landed[k], stream));
-    }
-    return (int)hipStreamSynchronize(stream);
+    auto run = [&]() -> int {
+        for (size_t i = 0; i < chunks; ++i) {
+            const int k = (int)(i % kRing);
+            const size_t n = std::min(kChunk, nbytes - i * kChunk);
+            if (i >= (size_t)kRing)  // the DMA that read this buffer kRing chunks ago must be over
+                NBH_TRY(hipEventSynchronize(ring->landed[k]));
+            p.crew->copy(ring->buf[k], (const char *)src + i * kChunk, n);
+            NBH_TRY(hipMemcpyAsync((char *)dst + i * kChunk, ring->buf[k], n, hipMemcpyHostToDevice, stream));
+            NBH_TRY(hipEventRecord(ring->landed[k], stream));
+        }
+        return 0;
+    };
+    rc = run();
+    // success or not, the ring is only handed to the next copy once every DMA that reads it is over
+    const int drained = (int)hipStreamSynchronize(stream);
+    return rc ? rc : drained;
 }

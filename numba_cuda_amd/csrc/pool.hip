@@ -23,52 +23,60 @@
 // class.  When hipMalloc runs out of memory, every idle block is returned to the
 // driver and the allocation retried once.
 #include "common.h"
+#include "pool_core.h"
+
+#include <pthread.h>
 
 #include <atomic>
 #include <map>
-#include <memory>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
 
 namespace {
 
-struct SharedEvent {
-    hipEvent_t ev = nullptr;
-    bool done = false;
-    ~SharedEvent()
+struct HipBackend {
+    using Event = hipEvent_t;
+    static bool event_record(Event *out, hipStream_t s)
     {
-        if (ev)
-            (void)hipEventDestroy(ev);
-    }
-    bool finished()
-    {
-        if (!done) {
-            const hipError_t e = hipEventQuery(ev);
-            if (e == hipSuccess)
-                done = true;
-            else if (e != hipErrorNotReady)
-                (void)hipGetLastError();
+        hipEvent_t ev = nullptr;
+        if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
         }
-        return done;
+        if (hipEventRecord(ev, s) != hipSuccess) {
+            (void)hipGetLastError();
+            (void)hipEventDestroy(ev);
+            return false;
+        }
+        *out = ev;
+        return true;
     }
+    static bool event_done(Event e)
+    {
+        const hipError_t rc = hipEventQuery(e);
+        if (rc == hipSuccess)
+            return true;
+        if (rc != hipErrorNotReady)
+            (void)hipGetLastError();
+        return false;
+    }
+    static void event_destroy(Event e) { (void)hipEventDestroy(e); }
+    static void device_synchronize() { (void)hipDeviceSynchronize(); }
+    static bool is_per_thread(hipStream_t s) { return s == hipStreamPerThread; }
+    static uint64_t thread_id() { return (uint64_t)pthread_self(); }
 };
-using EventRef = std::shared_ptr<SharedEvent>;
-
-struct StreamState {
-    bool used = false;  // work submitted since `last` was recorded
-    EventRef last;      // covers everything submitted before it
-};
+using Tracker = nbh_pool::Tracker<HipBackend, hipStream_t>;
 
 struct Block {
     void *ptr;
-    std::vector<EventRef> waits;
+    std::vector<Tracker::EventRef> waits;
 };
 
 struct DevicePool {
     std::map<size_t, std::vector<Block>> idle;  // size class -> blocks
     std::unordered_map<void *, size_t> live;    // handed out: ptr -> size class
-    std::unordered_map<hipStream_t, StreamState> streams;
+    Tracker tracker;
     size_t idle_bytes = 0, live_bytes = 0;
     uint64_t hits = 0, misses = 0;
 };
@@ -77,18 +85,7 @@ std::mutex g_mu;
 DevicePool g_pools[64];
 std::atomic<bool> g_enabled{false};  // set by the first nbh_pool_malloc
 
-size_t size_class(size_t n)
-{
-    if (n == 0)
-        n = 1;
-    if (n <= ((size_t)1 << 20))
-        return (n + 511) & ~(size_t)511;
-    size_t pow2 = (size_t)1 << 21;
-    while (pow2 < n)
-        pow2 <<= 1;
-    const size_t step = pow2 >> 4;  // 1/8 of the power of two below pow2
-    return (n + step - 1) / step * step;
-}
+using nbh_pool::size_class;
 
 int current_pool(DevicePool **out)
 {
@@ -98,19 +95,6 @@ int current_pool(DevicePool **out)
         return (int)hipErrorInvalidDevice;
     *out = &g_pools[dev];
     return 0;
-}
-
-bool ready(Block &b)
-{
-    for (size_t i = 0; i < b.waits.size();) {
-        if (b.waits[i]->finished()) {
-            b.waits[i] = b.waits.back();
-            b.waits.pop_back();
-        } else {
-            ++i;
-        }
-    }
-    return b.waits.empty();
 }
 
 // hipFree every idle block (they may still be waited on: hipFree itself waits).
@@ -133,7 +117,7 @@ void nbh_pool_note_stream(hipStream_t stream)
     if (current_pool(&p))
         return;
     std::lock_guard<std::mutex> lock(g_mu);
-    p->streams[stream].used = true;
+    p->tracker.note_stream(stream);
 }
 
 void nbh_pool_forget_stream(hipStream_t stream)
@@ -144,7 +128,7 @@ void nbh_pool_forget_stream(hipStream_t stream)
     if (current_pool(&p))
         return;
     std::lock_guard<std::mutex> lock(g_mu);
-    p->streams.erase(stream);  // blocks keep their own references to its events
+    p->tracker.forget_stream(stream);  // blocks keep their own references to its events
 }
 
 extern "C" {
@@ -163,7 +147,7 @@ int nbh_pool_malloc(void **ptr, size_t nbytes)
     if (it != p->idle.end()) {
         std::vector<Block> &blocks = it->second;
         for (size_t i = blocks.size(); i-- > 0;) {  // most recently freed first
-            if (ready(blocks[i])) {
+            if (Tracker::ready(blocks[i].waits)) {
                 void *got = blocks[i].ptr;
                 blocks[i] = std::move(blocks.back());
                 blocks.pop_back();
@@ -208,24 +192,7 @@ int nbh_pool_free(void *ptr)
     const size_t cls = it->second;
     p->live.erase(it);
     p->live_bytes -= cls;
-    Block b{ptr, {}};
-    for (auto &entry : p->streams) {
-        StreamState &st = entry.second;
-        if (st.used) {
-            auto ev = std::make_shared<SharedEvent>();
-            if (hipEventCreateWithFlags(&ev->ev, hipEventDisableTiming) != hipSuccess ||
-                hipEventRecord(ev->ev, entry.first) != hipSuccess) {
-                (void)hipGetLastError();
-                // cannot track this stream: fall back to what hipFree would have done
-                (void)hipDeviceSynchronize();
-                ev->done = true;
-            }
-            st.last = ev;
-            st.used = false;
-        }
-        if (st.last && !st.last->finished())
-            b.waits.push_back(st.last);
-    }
+    Block b{ptr, p->tracker.waits_for_a_free()};
     p->idle[cls].push_back(std::move(b));
     p->idle_bytes += cls;
     return 0;

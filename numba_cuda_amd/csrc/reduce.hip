@@ -22,7 +22,18 @@
 // is put in place with an agent-scope atomic EXCHANGE - a read-modify-write is carried
 // out where every XCD looks, and its result comes back from there - the wavefront
 // waits for that result, and only then takes its ticket with a relaxed agent-scope
-// atomic add.  (A written-through atomic store followed by a wait for its
+// atomic add.
+// THE INVARIANT THIS RESTS ON: on gfx942 / gfx950 the L2 caches of the eight XCDs are not
+// coherent with one another; agent-scope atomics are issued with the sc1 bit, which sends
+// them past the XCD's own L2 to the one place all XCDs share (LLVM's AMDGPU memory model
+// for gfx942 lowers every agent-scope atomicrmw and atomic load to an sc1 access for this
+// reason).  A returning atomic's result is produced there, after the new value is in
+// place, so (a) once the result is back the partial can be seen by an sc1 load from any
+// XCD, and (b) the finisher's sc1 loads cannot be served from a stale private L2.  What the
+// documentation does NOT promise is any order between two atomics to DIFFERENT addresses
+// that are merely issued one after the other - hence the wait for the result in between.
+// In the language-level memory model the relaxed accesses still form a race on the
+// partials; NBH_REDUCE_RELEASE_PUBLISH=1 builds the release/acquire protocol instead.  (A written-through atomic store followed by a wait for its
 // acknowledgement is not enough: the acknowledgement does not mean that the value is
 // where other XCDs read it.  With tickets and partials in different pages a ticket was
 // seen to overtake its partial, one wrong sum in some 10^4 closings; the exchange costs
@@ -50,6 +61,12 @@ constexpr size_t kHeaderBytes = 256;  // ticket counter, padded to its own cache
 constexpr size_t kScratchBytes = kHeaderBytes + sizeof(uint64_t) * kMaxGrid;
 constexpr int kGridPerCU = 2;
 constexpr int kUnroll = 4;
+// Build with -DNBH_REDUCE_RELEASE_PUBLISH=1 to publish partials the slow, by-the-book way
+// (see "Publishing a partial" above): the reference point when the fast protocol is in doubt.
+#ifndef NBH_REDUCE_RELEASE_PUBLISH
+#define NBH_REDUCE_RELEASE_PUBLISH 0
+#endif
+constexpr bool kReleasePublish = NBH_REDUCE_RELEASE_PUBLISH != 0;
 
 // ---- complex elements -------------------------------------------------------------
 // An aggregate (it lives in unions with raw packets).  Multiplication is the plain
@@ -331,17 +348,27 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
     Word *partials = reinterpret_cast<Word *>(partials_raw);
     if (tid == 0) {
         const Image img = WordsOf<A>::pack(total);
-        Word before[kWords];
+        unsigned t;
+        if constexpr (kReleasePublish) {
+            // the textbook protocol: ordinary stores, then a ticket drawn with release
+            // semantics at agent scope (writes this XCD's L2 back before the ticket moves)
 #pragma unroll
-        for (int w = 0; w < kWords; ++w)
-            before[w] = __hip_atomic_exchange(&partials[(int64_t)blockIdx.x * kWords + w], img.w[w], __ATOMIC_RELAXED,
-                                              __HIP_MEMORY_SCOPE_AGENT);
-        // the results of the exchanges come from where every XCD looks: once they are
-        // back, the partial is in place and the ticket may be drawn
+            for (int w = 0; w < kWords; ++w)
+                partials[(int64_t)blockIdx.x * kWords + w] = img.w[w];
+            t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            Word before[kWords];
 #pragma unroll
-        for (int w = 0; w < kWords; ++w)
-            asm volatile("" ::"v"(before[w]) : "memory");
-        unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int w = 0; w < kWords; ++w)
+                before[w] = __hip_atomic_exchange(&partials[(int64_t)blockIdx.x * kWords + w], img.w[w],
+                                                  __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // the results of the exchanges come from where every XCD looks: once they are
+            // back, the partial is in place and the ticket may be drawn
+#pragma unroll
+            for (int w = 0; w < kWords; ++w)
+                asm volatile("" ::"v"(before[w]) : "memory");
+            t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         last_block = (t == gridDim.x - 1);
         if (last_block)  // every partial has been published: drop stale cache lines once
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -462,7 +489,7 @@ int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, 
         ((uintptr_t)scratch) % 8 != 0)
         return (int)hipErrorInvalidValue;
     hipStream_t s = nbh_hip_stream(stream);
-    nbh_pool_note_stream(s);
+    nbh_stream_report report(s);
     switch (dtype) {
     case NBH_I8: return launch_op<int8_t>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_I16: return launch_op<int16_t>(op, in, n, in_stride, init, out, scratch, s);

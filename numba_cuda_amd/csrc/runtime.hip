@@ -194,7 +194,7 @@ static int copy(void *dst, const void *src, size_t nbytes, hipMemcpyKind kind, n
 {
     if (nbytes == 0)
         return 0;
-    nbh_pool_note_stream(nbh_hip_stream(stream));
+    nbh_stream_report report(nbh_hip_stream(stream));
     if (stream)
         return (int)hipMemcpyAsync(dst, src, nbytes, kind, nbh_hip_stream(stream));
     return (int)hipMemcpy(dst, src, nbytes, kind);
@@ -204,7 +204,7 @@ static int copy(void *dst, const void *src, size_t nbytes, hipMemcpyKind kind, n
 // the call either way).
 int nbh_memcpy_h2d(void *dst, const void *src, size_t nbytes, nbh_stream_t stream)
 {
-    nbh_pool_note_stream(nbh_hip_stream(stream));
+    nbh_stream_report report(nbh_hip_stream(stream));
     const int rc = nbh_staged_h2d(dst, src, nbytes, nbh_hip_stream(stream));
     if (rc >= 0)
         return rc;
@@ -212,7 +212,7 @@ int nbh_memcpy_h2d(void *dst, const void *src, size_t nbytes, nbh_stream_t strea
 }
 int nbh_memcpy_d2h(void *dst, const void *src, size_t nbytes, nbh_stream_t stream)
 {
-    nbh_pool_note_stream(nbh_hip_stream(stream));
+    nbh_stream_report report(nbh_hip_stream(stream));
     const int rc = nbh_staged_d2h(dst, src, nbytes, nbh_hip_stream(stream));
     if (rc >= 0)
         return rc;
@@ -251,7 +251,7 @@ int nbh_memset8(void *dst, int byte, size_t nbytes, nbh_stream_t stream)
 {
     if (nbytes == 0)
         return 0;
-    nbh_pool_note_stream(nbh_hip_stream(stream));
+    nbh_stream_report report(nbh_hip_stream(stream));
     if (stream)
         return (int)hipMemsetAsync(dst, byte, nbytes, nbh_hip_stream(stream));
     return (int)hipMemset(dst, byte, nbytes);

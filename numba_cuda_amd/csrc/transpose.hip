@@ -508,7 +508,7 @@ extern "C" int nbh_transpose(const void *in, void *out, int64_t rows, int64_t co
     if (!in || !out)
         return (int)hipErrorInvalidValue;
     hipStream_t s = nbh_hip_stream(stream);
-    nbh_pool_note_stream(s);
+    nbh_stream_report report(s);
 
     // largest power of two (<= 16) that divides the item size, every stride and
     // both base addresses: the widest access that is aligned everywhere

@@ -796,7 +796,7 @@ int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t 
         if (rc)
             return rc;
     }
-    nbh_pool_note_stream(nbh_hip_stream(stream));
+    nbh_stream_report report(nbh_hip_stream(stream));
     using VT = typename Gen::value_type;
     const bool on_lines = ((uintptr_t)out % 128 == 0) && ((uint64_t)count * sizeof(VT)) % 128 == 0;
     // Lines per generator and round (measured, 2^24 generators, uniform draws): two lines
@@ -888,7 +888,7 @@ int nbh_xoro_one(void *state, int kind, void *out, nbh_stream_t stream)
     hipLaunchKernelGGL(one_generator_kernel, dim3(1), dim3(64), 0, nbh_hip_stream(stream), (uint64_t *)state, kind,
                        out, log_table);
     const int rc = nbh_launch_status();
-    nbh_pool_note_stream(nbh_hip_stream(stream));
+    nbh_stream_report report(nbh_hip_stream(stream));
     return rc;
 }
 
@@ -916,7 +916,7 @@ int nbh_xoro_init_states(void *states, int64_t n, uint64_t seed, uint64_t subseq
     if (rc)
         return rc;
     hipStream_t hs = nbh_hip_stream(stream);
-    nbh_pool_note_stream(hs);
+    nbh_stream_report report(hs);
     if (n >= kTablesFrom) {
         // one workgroup of 16 wavefronts per 65536 states, lookup tables in LDS
         const int64_t per_block = (int64_t)(kTabBlock / 64) * 64 * kInitSteps;
