@@ -32,21 +32,21 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E published peak
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (see profiles/); filled in per workload once measured, else None
 MEASURED_TRAFFIC = {
-    # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 780 027 B fetched + 32 832 B written
-    "reduce_f32_sum": 1073812859,
+    # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 777 931 B fetched + 32 823 B written
+    "reduce_f32_sum": 1073810755,
     # profiles/copy_flat_f32_2p28.txt: the calibration kernel itself
     "copy_f32": 2147483648,
-    # profiles/transpose_packets_f32_16384sq.txt: 1 073 769 401 B fetched + 1 074 524 157 B written
-    "transpose_f32": 2148293558,
+    # profiles/transpose_packets_f32_16384sq.txt: 1 073 772 464 B fetched + 1 073 962 931 B written
+    "transpose_f32": 2147735395,
     # profiles/xoroshiro_fill_and_init_2p24.txt: 268 618 773 B fetched + 4 563 547 721 B written
     "rng_uniform_f32": 4832166494,
-    # profiles/transpose_sheared_f64_12345x6789.txt: 1 026 969 245 B fetched + 670 744 593 B written
-    "transpose_f64": 1697713838,
+    # profiles/transpose_sheared_f64_12345x6789.txt: 1 083 619 701 B fetched + 670 476 024 B written
+    "transpose_f64": 1754095725,
     # profiles/hbm_counters_other_workloads.txt
     "reduce_f32_max": 1073822046,
     "reduce_f64_sum": 1073820062,
     "reduce_i64_sum": 2147534810,
-    "transpose_i16": 1074008367,
+    "transpose_i16": 1073845912,
     "rng_normal_f64": 2684437180,
     "rng_init": 269594109,
 }
