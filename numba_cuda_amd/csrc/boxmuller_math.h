@@ -4,6 +4,7 @@
 //   bm_log_f32(u)  natural logarithm of a float32 in (0, 1] (any positive normal
 //                  float32 works), evaluated in double; u == 0 gives -infinity.
 //   bm_cos_2pi(x)  cosine of a double in [0, 6.2832], i.e. of 2*pi*u.
+//   bm_sqrt_pos(a) square root for the range that occurs.
 //
 // The general-purpose library routines spend most of their time on cases that
 // cannot occur here (subnormals, huge arguments, Payne-Hanek reduction): on
@@ -167,6 +168,29 @@ BM_FN double bm_cos_2pi(double x, const LogTable *__restrict__ tab)
     const double pick = base + __builtin_fma(factor, q, tail);
     // cos(n*pi/2 + y): n&3 = 0: cos y, 1: -sin y, 2: -cos y, 3: sin y
     return (((n + 1) & 2) != 0) ? -pick : pick;
+}
+
+// Square root of -2 log(u): zero, +infinity or a double in [2^-22, 210] - never
+// subnormal, so the range scaling the general routine wraps around the same steps (two
+// ldexp, a compare, two selects) is left out.  Reciprocal square root estimate, one
+// coupled Newton step on (g, h) ~ (sqrt a, 1 / (2 sqrt a)), two corrections of g.
+BM_FN double bm_sqrt_pos(double a)
+{
+#ifdef __HIP_DEVICE_COMPILE__
+    const double y = __builtin_amdgcn_rsq(a);
+    double g = a * y;
+    double h = 0.5 * y;
+    const double r = __builtin_fma(-h, g, 0.5);
+    g = __builtin_fma(g, r, g);
+    h = __builtin_fma(h, r, h);
+    double d = __builtin_fma(-g, g, a);
+    g = __builtin_fma(d, h, g);
+    d = __builtin_fma(-g, g, a);
+    g = __builtin_fma(d, h, g);
+    return (a == 0.0 || a == HUGE_VAL) ? a : g;
+#else
+    return std::sqrt(a);
+#endif
 }
 
 }  // namespace bm

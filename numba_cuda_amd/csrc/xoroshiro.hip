@@ -414,7 +414,7 @@ struct NormalF64 {
         const float u2 = UniformF32::draw(s0, s1);
         const double two_pi = 6.283185307179586;
         const float lg = (float)bm::bm_log_f32(u1, tab);
-        const double r = sqrt(-2.0 * (double)lg);
+        const double r = bm::bm_sqrt_pos(-2.0 * (double)lg);
         const double c = bm::bm_cos_2pi(two_pi * (double)u2, tab);
         return r * c;
     }
