@@ -194,6 +194,35 @@ int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, 
 int nbh_reduce_noalloc(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init,
                        void *out, nbh_stream_t stream);
 
+/* Reductions with a binary operation supplied as source text.  Stands where the
+ * reference's JIT compiles an arbitrary Python functor for the reduction kernels
+ * (kernels/reduction.py:15-20, :175-192 Reduce._compile).
+ *
+ * nbh_reduce_compile builds, with the HIP run-time compiler (libhiprtc.so, loaded on
+ * first use), the kernels for
+ *     __device__ T nbh_op(T a, T b) { <body> }
+ * where T is the C type of `dtype` (NBH_I8 .. NBH_F64 and NBH_F16; not the complex types)
+ * and `body` is C++ that returns the combined value.  Available to the body: the HIP
+ * device math functions, nbh_i64 / nbh_u64 (64-bit integer types), nbh_floordiv(x, y) and
+ * nbh_mod(x, y) with Python's rounding for nbh_i64, nbh_u64, float and double, and
+ * nbh_ipow(x, e).  Needs no device.  On failure the compiler's messages are in `log`
+ * (NUL-terminated, cut to log_bytes) and the result is hipErrorInvalidSource (300), or
+ * hipErrorSharedObjectInitFailed (303) when the compiler library is absent.
+ * `*op` stays valid until nbh_reduce_op_free(op); it may be used from any thread and on
+ * any device (each device loads its module at its first call). */
+int nbh_reduce_compile(int dtype, const char *body, void **op, char *log, size_t log_bytes);
+int nbh_reduce_op_dtype(const void *op);
+int nbh_reduce_op_free(void *op);
+
+/* out[0] = nbh_op(... nbh_op(nbh_op(in[0], in[1]), in[2]) ..., init) in SOME order of
+ * association: every element and `init` enter exactly once, n applications for n
+ * elements, so the result equals the reference's (kernels/reduction.py:194-265) for every
+ * operation that is associative and commutative - the same condition the reference's own
+ * tree imposes.  Arguments as for nbh_reduce (`scratch` is the same buffer; its ticket is
+ * left alone).  Two launches on `stream`, fully asynchronous. */
+int nbh_reduce_custom(void *op, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
+                      void *scratch, size_t scratch_bytes, nbh_stream_t stream);
+
 /* ---- transpose ------------------------------------------------------------ */
 
 /* kernels/transpose.py:10-65 transpose(a, b): out[j, i] = in[i, j] for a

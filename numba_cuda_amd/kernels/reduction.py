@@ -1,12 +1,17 @@
 """`Reduce`: full reduction of a 1-d array with a binary operator.
 
 Drop-in for numba_cuda/numba/cuda/kernels/reduction.py:169-265.  The reference
-JIT-compiles the Python functor into a three-launch tree reduction; here the
-functor is *recognised* as one of the operators that have hand-written HIP
-kernels (a + b, a * b, max(a, b), min(a, b), and a & b, a | b, a ^ b on integers) and a single launch of
-nbh_reduce does the work.  Element types: the integers, booleans, float16 (accumulated in
-float16, as the reference's JIT does), float32, float64, complex64 and complex128.  Anything else raises NotImplementedError - there is
-no slower path to fall back to.
+JIT-compiles the Python functor into a three-launch tree reduction.  Here the functor is
+first *recognised*: a + b, a * b, max(a, b), min(a, b), and a & b, a | b, a ^ b on
+integers have hand-written HIP kernels, and a single launch of nbh_reduce does the work.
+Element types on that path: the integers, booleans, float16 (accumulated in float16, as
+the reference's JIT does), float32, float64, complex64 and complex128.
+
+Any other functor is translated (kernels/functor.py: run on recording stand-ins, typed
+with the JIT's rules, written out as C++) and compiled for the device at run time, once
+per functor and element type; nbh_reduce_custom then runs it in two launches.  Element
+types there: integers, booleans and the real floating-point types.  What cannot be
+translated raises NotImplementedError - there is no host fallback.
 """
 
 import operator
@@ -16,6 +21,7 @@ import numpy as np
 from numba_cuda_amd import _lib
 from numba_cuda_amd.cudadrv import devicearray, devices
 from numba_cuda_amd.cudadrv import driver as _driver
+from numba_cuda_amd.kernels import functor as _functor
 
 
 class _Sym:
@@ -175,13 +181,24 @@ class Reduce:
         try:
             self._op = self._cache[functor]
         except (KeyError, TypeError):
-            self._op = classify_functor(functor)
+            try:
+                self._op = classify_functor(functor)
+            except NotImplementedError:
+                # not one of the operators with kernels of their own: translate it
+                try:
+                    self._op = _functor.trace(functor)
+                except NotImplementedError as why:
+                    raise NotImplementedError(
+                        "Reduce could not translate %r for the device: %s.  Translated are arithmetic, "
+                        "comparisons, conditionals and math functions of the two operands." % (functor, why)) from None
             try:
                 self._cache[functor] = self._op
             except TypeError:
                 pass
-        self._opcode = _lib.OP_CODES[self._op]
+        self._custom = not isinstance(self._op, str)
+        self._opcode = None if self._custom else _lib.OP_CODES[self._op]
         self._codes = {}    # dtype -> (operator code, element code), filled once the pairing is checked
+                            # (translated functors: dtype -> handle of the compiled operation)
 
     def _codes_for(self, dtype):
         """(operator code, element code) nbh_reduce is called with for arrays of `dtype`."""
@@ -229,6 +246,8 @@ class Reduce:
         n = arr.size
         if n < 1:
             return dtype.type(init)          # `res` is left untouched, as in the reference
+        if self._custom:
+            return self._call_translated(arr, dtype, n, res, init, stream)
 
         codes = self._codes.get(dtype)
         if codes is None:
@@ -288,6 +307,65 @@ class Reduce:
             return cell[1][:dtype.itemsize].view(dtype)[0]
         finally:
             ctx.give_back_result_cell(cell)
+
+
+    def _call_translated(self, arr, dtype, n, res, init, stream):
+        """The same call for a functor that was translated and compiled at run time."""
+        ctx = devices.get_context()              # also loads the library on the first call
+        handle = self._codes.get(dtype)
+        if handle is None:
+            handle = self._codes[dtype] = compile_translated(self._op, dtype)
+        if not _driver.is_device_memory(arr):
+            arr, _ = devicearray.auto_device(arr, stream=stream)
+        in_ptr = arr.device_ctypes_pointer.value
+        hstream = _driver._stream_handle(stream)
+        scratch = ctx.reduce_scratch(hstream)
+        init_ptr = _init_buffer(dtype, init)
+        lib = _driver.driver.lib
+        if res is not None:
+            if res.dtype != dtype:
+                raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
+            rc = lib.nbh_reduce_custom(handle, in_ptr, n, arr.strides[0], init_ptr, res.device_ctypes_pointer.value,
+                                       scratch[0], scratch[1], hstream or None)
+            if rc:
+                _driver.driver.check("nbh_reduce_custom", rc)
+            return None
+        cell = ctx.take_result_cell()
+        try:
+            rc = lib.nbh_reduce_custom(handle, in_ptr, n, arr.strides[0], init_ptr, cell[0],
+                                       scratch[0], scratch[1], hstream or None)
+            if rc:
+                _driver.driver.check("nbh_reduce_custom", rc)
+            _driver.driver.nbh_stream_synchronize(hstream or None)
+            return cell[1][:dtype.itemsize].view(dtype)[0]
+        finally:
+            ctx.give_back_result_cell(cell)
+
+
+# (body, element code) -> handle from nbh_reduce_compile, kept for the life of the process
+_COMPILED = {}
+
+
+def compile_translated(expr, dtype):
+    """Handle of the compiled operation for an expression tree and an element type
+    (what Reduce._compile, kernels/reduction.py:182-190, is in the reference)."""
+    import ctypes
+    body = _functor.body_for(expr, dtype)
+    code = _DTYPE_CODE[np.dtype(np.uint8)] if dtype == _BOOL else _DTYPE_CODE.get(dtype)
+    if code is None or dtype.kind == "c":
+        raise NotImplementedError("Reduce with a general functor does not support dtype %s" % dtype)
+    key = (body, code)
+    handle = _COMPILED.get(key)
+    if handle is None:
+        lib = _driver.driver.lib
+        out = ctypes.c_void_p()
+        log = ctypes.create_string_buffer(8192)
+        rc = lib.nbh_reduce_compile(code, body.encode(), ctypes.byref(out), log, len(log))
+        if rc:
+            raise RuntimeError("compiling the functor for %s failed (error %d)\n%s\n-- generated code --\n%s"
+                               % (dtype, rc, log.value.decode(errors="replace"), body))
+        handle = _COMPILED[key] = out.value
+    return handle
 
 
 _Stream = _driver.Stream

@@ -4,6 +4,7 @@ Test infrastructure: see the package docstring.
 """
 
 import ctypes
+import math
 import os
 import subprocess
 
@@ -173,6 +174,176 @@ def fold(op, a, init=0):
 def tree(op, a, init=0):
     """The association order of the reference's CUDA kernels."""
     return _reduce("tree", op, a, init)
+
+
+# ---- general functors --------------------------------------------------------------
+# Pure Python: for small inputs only.  Pinned by tests/test_oracle_functors.py: with
+# a + b, a * b, max and min these give, bit for bit, what the C restatements orc_fold_* /
+# orc_tree_* above give (float32 sums included, which are sensitive to the order), and the
+# typing is checked against closed forms on wrapped integers.
+
+def typed_functor(functor, dtype):
+    """functor(a, b) on elements of `dtype`, converted back to `dtype`, the way the
+    reference's JIT types it (kernels/reduction.py:15-20 compiles the functor for the
+    element type; the kernels store every intermediate result in arrays of that type,
+    :32-37, :96):
+      integers  operands enter as exact integers (the JIT computes in 64 bits: equal
+                after the final wrap for + - * & | ^ and for everything else as long as
+                no intermediate value leaves 64 bits), the result wraps to the type
+      booleans  operands are bools, the result is `!= 0`
+      float64   Python floats are float64
+      float32 / float16  NumPy scalars of that type.  A Python float constant in the
+                functor makes the JIT compute that step in float64, NumPy keeps it in
+                the narrow type: such functors agree to the narrow type's rounding."""
+    dtype = np.dtype(dtype)
+    if dtype.kind in "iu":
+        bits = 8 * dtype.itemsize
+        mask, top = (1 << bits) - 1, 1 << (bits - 1)
+
+        def on_integers(a, b):
+            r = functor(int(a), int(b))
+            if isinstance(r, (float, np.floating)):
+                r = int(r)                   # conversion of a float result: towards zero
+            r = int(r) & mask
+            if dtype.kind == "i" and r >= top:
+                r -= 1 << bits
+            return dtype.type(r)
+        return on_integers
+    if dtype.kind == "b":
+        return lambda a, b: np.bool_(bool(functor(bool(a), bool(b))))
+    if dtype == np.dtype(np.float64):
+        return lambda a, b: np.float64(functor(float(a), float(b)))
+    scalar = dtype.type
+    narrow = _with_narrow_math(functor, scalar)
+
+    def on_narrow_floats(a, b):
+        with np.errstate(all="ignore"):
+            return scalar(narrow(scalar(a), scalar(b)))
+    return on_narrow_floats
+
+
+class _NarrowMath:
+    """`math` whose functions return the narrow float type when they are given one: the
+    JIT types math.exp(float32) as float32 (the float32 routine), while Python's math
+    module works in float64 - one rounding of the float64 value stands in for it."""
+
+    def __init__(self, scalar):
+        self._scalar = scalar
+
+    def wrap(self, fn):
+        scalar = self._scalar
+
+        def narrow(*args):
+            out = fn(*[float(x) if isinstance(x, np.floating) else x for x in args])
+            if isinstance(out, float) and any(isinstance(x, scalar) for x in args):
+                return scalar(out)
+            return out
+        return narrow
+
+    def __getattr__(self, name):
+        value = getattr(math, name)
+        return self.wrap(value) if callable(value) else value
+
+
+def _with_narrow_math(functor, scalar):
+    import types
+    if not isinstance(functor, types.FunctionType):
+        return functor
+    proxy = _NarrowMath(scalar)
+
+    def swap(value):
+        if value is math:
+            return proxy
+        if isinstance(value, types.BuiltinFunctionType) and getattr(math, value.__name__, None) is value:
+            return proxy.wrap(value)
+        return value
+    new_globals = dict(functor.__globals__)
+    for name in functor.__code__.co_names:
+        if name in new_globals:
+            new_globals[name] = swap(new_globals[name])
+    closure = functor.__closure__
+    if closure:
+        closure = tuple(types.CellType(swap(c.cell_contents)) for c in closure)
+    clone = types.FunctionType(functor.__code__, new_globals, functor.__name__, functor.__defaults__, closure)
+    clone.__kwdefaults__ = functor.__kwdefaults__
+    return clone
+
+
+def functor_fold(functor, a, init=0):
+    """simulator/reduction.py:7-19: functools.reduce(functor, a, init), typed."""
+    a = np.asarray(a)
+    f = typed_functor(functor, a.dtype)
+    acc = a.dtype.type(init)
+    for x in a:
+        acc = f(acc, x)
+    return acc
+
+
+_WARP, _NWARPS, _MAXGRID = 32, 4, 64
+
+
+def functor_tree(functor, a, init=0):
+    """kernels/reduction.py:194-265 with the device functions at :22-166, in the
+    association order a CUDA run uses - the same walk as orc_tree_* in oracle.c, with a
+    Python functor in place of the operator."""
+    a = np.asarray(a)
+    f = typed_functor(functor, a.dtype)
+    init = a.dtype.type(init)
+    n = a.size
+    if n < 1:
+        return init
+    block = _WARP * _NWARPS
+
+    def warp_tree(v):                        # :22-41, one full warp
+        v = list(v)
+        width = _WARP // 2
+        while width:
+            for lane in range(width):
+                v[lane] = f(v[lane], v[lane + width])
+            width //= 2
+        return v[0]
+
+    def one_block(items):                    # :99-141, fewer than 128 lanes
+        m = len(items)
+        results = []
+        for w in range((m + _WARP - 1) // _WARP):
+            if (w + 1) * _WARP < m:
+                results.append(warp_tree(items[w * _WARP:(w + 1) * _WARP]))
+            else:
+                acc = items[w * _WARP]
+                for x in items[w * _WARP + 1:m]:
+                    acc = f(acc, x)
+                results.append(acc)
+        r = results[0]
+        for x in results[1:]:
+            r = f(r, x)
+        return r
+
+    size_full = (n // block) * block
+    grid = min(size_full // block, _MAXGRID)
+    stride = block * grid
+    partials = []
+    for blk in range(grid):                  # :43-97, :233-248
+        per_warp = []
+        for w in range(_NWARPS):
+            lanes = []
+            for lane in range(_WARP):
+                g = blk * block + w * _WARP + lane
+                acc = a[g]
+                for i in range(g + stride, size_full, stride):
+                    acc = f(acc, a[i])
+                lanes.append(acc)
+            per_warp.append(warp_tree(lanes))
+        partials.append(f(f(per_warp[0], per_warp[2]), f(per_warp[1], per_warp[3])))
+    if grid:
+        partials[0] = f(partials[0], init)   # :163-164
+    if n - size_full:                        # :250-254
+        partials.append(one_block(list(a[size_full:])))
+        if not grid:
+            partials[0] = f(partials[0], init)
+    if len(partials) > 1:                    # :256-258
+        partials[0] = one_block(partials)
+    return partials[0]
 
 
 def sum_exact(a):

@@ -62,7 +62,7 @@ def test_only_1d_and_unknown_functor():
     with pytest.raises(TypeError, match="only support 1D array"):
         sum_reduce(np.zeros((2, 2)))
     with pytest.raises(NotImplementedError):
-        cuda.Reduce(lambda a, b: a - b)
+        cuda.Reduce(lambda a, b: int(a) - b)
 
 
 def test_size_argument_and_offset_views():

@@ -1,0 +1,220 @@
+"""Reduce with functors that are translated and compiled at run time (HIP path through
+nbh_reduce_compile / nbh_reduce_custom), against the oracle.
+
+Oracle: oracle.cref.functor_tree - the functor itself, typed as the reference's JIT types
+it, applied in the association order of the reference's kernels - for sizes it finishes
+in seconds; closed forms at 2^24 elements.  Every functor here is associative and
+commutative on its operands, so the order of association cannot change an integer or
+boolean result: those are compared bit for bit.  Floats: `largest_magnitude` selects an
+element (bit for bit); sums and the hypot and log-sum-exp folds accumulate a rounding (and
+a library call) per application in an order that differs from the oracle's: tolerance
+4 n eps, relative to the sum of magnitudes for sums and to the result otherwise (written
+at the assertion).
+"""
+
+import threading
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import numba_cuda_amd as cuda
+from numba_cuda_amd.kernels import reduction
+from oracle import cref
+from tests import functor_cases as FC
+
+FOLDS = [c for c in FC.CASES if c.fold]
+SIZES = [1, 2, 63, 64, 65, 255, 256, 257, 1023, 4099, 70001]
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _check(case, dtype, got, want, n, data):
+    dtype = np.dtype(dtype)
+    assert isinstance(got, dtype.type), (case, dtype, type(got))
+    if dtype.kind != "f" or case.selects:
+        assert got.tobytes() == want.tobytes(), (case, dtype, n, got, want)
+    else:
+        # sums: against the sum of magnitudes; the other folds: against the result
+        eps = np.finfo(dtype).eps
+        scale = float(np.abs(data.astype(np.float64)).sum()) + n if case.name == "sum_plus_one" else abs(float(want))
+        assert abs(float(got) - float(want)) <= 4 * max(n, 8) * eps * scale, (case, dtype, n, got, want)
+
+
+@pytest.mark.parametrize("case", FOLDS, ids=repr)
+def test_folds_against_the_reference_order(case):
+    red = cuda.Reduce(case.functor)
+    for dtype in case.dtypes:
+        for n in SIZES:
+            _say(case, dtype, n)
+            data = case.operands(dtype, n, n)
+            want = cref.functor_tree(case.functor, data, case.init)
+            _check(case, dtype, red(data, init=case.init), want, n, data)
+
+
+def _wrap(value, dtype):
+    info = np.iinfo(dtype)
+    bits = 8 * np.dtype(dtype).itemsize
+    value &= (1 << bits) - 1
+    if info.min < 0 and value >= 1 << (bits - 1):
+        value -= 1 << bits
+    return np.dtype(dtype).type(value)
+
+
+def test_closed_forms_at_2p24():
+    n = 1 << 24
+    rng = np.random.default_rng(24)
+    for dtype in (np.int32, np.uint16, np.int64, np.uint64):
+        info = np.iinfo(dtype)
+        data = rng.integers(info.min, info.max, n, dtype=dtype, endpoint=True)
+        d = cuda.to_device(data)
+        _say("sum_plus_one", np.dtype(dtype))
+        got = cuda.Reduce(FC.BY_NAME["sum_plus_one"].functor)(d, init=7)
+        total = int(np.sum(data.astype(np.uint64), dtype=np.uint64))       # modulo 2^64
+        assert got == _wrap(total + 7 + n, dtype)
+        _say("xor_and_flip", np.dtype(dtype))
+        got = cuda.Reduce(FC.BY_NAME["xor_and_flip"].functor)(d, init=5)
+        assert got == _wrap(int(np.bitwise_xor.reduce(data)) ^ 5 ^ (n & 1), dtype)
+        _say("one_plus_products", np.dtype(dtype))
+        got = cuda.Reduce(FC.BY_NAME["one_plus_products"].functor)(d, init=2)
+        prod = int(np.multiply.reduce(data.astype(np.uint64) + np.uint64(1), dtype=np.uint64))       # wraps modulo 2^64
+        assert got == _wrap(prod * 3 - 1, dtype)
+    # saturation and the modulus
+    small = rng.integers(0, 40, n, dtype=np.int32)
+    assert cuda.Reduce(FC.BY_NAME["saturating_sum"].functor)(small, init=3) == 1000
+    assert cuda.Reduce(FC.BY_NAME["saturating_sum"].functor)(small[:20], init=3) == min(1000, int(small[:20].sum()) + 3)
+    residues = rng.integers(0, 1000003, n, dtype=np.int64)
+    assert cuda.Reduce(FC.BY_NAME["sum_modulo_prime"].functor)(residues, init=11) == (int(residues.sum()) + 11) % 1000003
+    # floats
+    for dtype, tol in ((np.float32, 1e-4), (np.float64, 1e-11)):
+        x = (rng.standard_normal(n) * 100).astype(dtype)
+        d = cuda.to_device(x)
+        got = cuda.Reduce(FC.BY_NAME["largest_magnitude"].functor)(d, init=0)
+        assert abs(got) == np.abs(x).max() and got in x and isinstance(got, dtype)
+        got = cuda.Reduce(FC.BY_NAME["hypot_math"].functor)(d, init=0)
+        want = np.sqrt(np.sum(x.astype(np.float64) ** 2))
+        assert abs(got - want) <= tol * want, (dtype, got, want)      # tolerance: 1e-4 / 1e-11 relative at 2^24
+    flags = rng.integers(0, 2, n).astype(np.bool_)
+    got = cuda.Reduce(FC.BY_NAME["different"].functor)(flags, init=False)
+    assert got == bool(flags.sum() & 1) and isinstance(got, np.bool_)
+
+
+def test_float16_and_booleans():
+    rng = np.random.default_rng(16)
+    x = (rng.standard_normal(5000) * 100).astype(np.float16)
+    x[1234] = np.float16(-60000)
+    got = cuda.Reduce(FC.BY_NAME["largest_magnitude"].functor)(x)
+    assert got == np.float16(-60000) and isinstance(got, np.float16)
+    for name in ("different", "both_or_neither", "sum_plus_one"):
+        case = FC.BY_NAME[name]
+        for n in (1, 7, 1000, 4097):
+            flags = case.operands("bool", n, n)
+            want = cref.functor_tree(case.functor, flags, case.init)
+            got = cuda.Reduce(case.functor)(flags, init=case.init)
+            assert got == want and isinstance(got, np.bool_), (name, n)
+
+
+def test_views_res_streams_and_size():
+    case = FC.BY_NAME["sum_plus_one"]
+    red = cuda.Reduce(case.functor)
+    rng = np.random.default_rng(3)
+    base = rng.integers(-1000, 1000, 100003).astype(np.int32)
+    d = cuda.to_device(base)
+
+    def expect(view, init=0):
+        return np.int32(int(view.astype(np.int64).sum()) + init + view.size)
+    assert red(d) == expect(base)
+    assert red(d, size=1000, init=5) == expect(base[:1000], 5)
+    for view_of in (lambda a: a[1:], lambda a: a[3:-5], lambda a: a[::3], lambda a: a[::-1], lambda a: a[7::-2],
+                    lambda a: a[4:4 + 4096]):
+        _say("view", view_of(base).shape, view_of(base).strides)
+        assert red(view_of(d)) == expect(view_of(base))
+    # result into device memory, on a stream, nothing comes back until asked
+    stream = cuda.stream()
+    res = cuda.device_array(3, np.int32)
+    res.copy_to_device(np.array([-1, -2, -3], np.int32))
+    assert red(d, res=res[1:], init=2, stream=stream) is None
+    stream.synchronize()
+    assert list(res.copy_to_host()) == [-1, expect(base, 2), -3]
+    with pytest.raises(TypeError, match="dtype"):
+        red(d, res=cuda.device_array(1, np.int64))
+    with pytest.raises(TypeError, match="1D"):
+        red(np.zeros((2, 2), np.int32))
+    # empty input: init, converted, the device is not asked
+    assert red(np.zeros(0, np.int16), init=9) == 9
+    # init takes part exactly once
+    assert red(np.array([5], np.int32), init=100) == 106
+    assert red(np.array([5, 6], np.int32), init=100) == 113
+
+
+def test_compiled_once_per_functor_and_type():
+    def functor(a, b):
+        return a + b + 2
+    before = len(reduction._COMPILED)
+    red = cuda.Reduce(functor)
+    assert red(np.arange(10, dtype=np.int32)) == 45 + 20
+    assert len(reduction._COMPILED) == before + 1
+    assert cuda.Reduce(functor)(np.arange(10, dtype=np.int32), init=1) == 45 + 21       # same functor: cached
+    assert len(reduction._COMPILED) == before + 1
+    assert red(np.arange(10, dtype=np.float64)) == 65.0                                  # another type: another build
+    assert len(reduction._COMPILED) == before + 2
+    # an equal body from another functor object shares the build
+    assert cuda.Reduce(lambda x, y: x + y + 2)(np.arange(4, dtype=np.int32)) == 6 + 8
+    assert len(reduction._COMPILED) == before + 2
+    # the decorator form of the reference
+    @cuda.reduce
+    def plus_three(a, b):
+        return a + b + 3
+    assert plus_three(np.arange(4, dtype=np.int64)) == 6 + 12
+
+
+def test_interleaved_with_the_kernels_of_the_standard_operators():
+    """Both kinds of calls share one scratch buffer per stream; the translated kernels
+    must leave the ticket of the single-launch kernels alone."""
+    rng = np.random.default_rng(8)
+    data = rng.integers(-100, 100, 1 << 20).astype(np.int64)
+    d = cuda.to_device(data)
+    plain = cuda.Reduce(lambda a, b: a + b)
+    custom = cuda.Reduce(lambda a, b: a + b + 1)
+    total = int(data.sum())
+    for _ in range(5):
+        assert plain(d) == total
+        assert custom(d) == total + data.size
+        assert plain(d, init=3) == total + 3
+
+
+def test_threads_on_their_own_streams():
+    case = FC.BY_NAME["xor_and_flip"]
+    red = cuda.Reduce(case.functor)
+    rng = np.random.default_rng(12)
+    arrays = [rng.integers(0, 2**31, 200000 + 1000 * k).astype(np.int32) for k in range(4)]
+    wants = [np.int32(int(np.bitwise_xor.reduce(a)) ^ (a.size & 1)) for a in arrays]
+    errors = []
+
+    def work(k):
+        try:
+            cuda.select_device(0)
+            d = cuda.to_device(arrays[k])
+            s = cuda.stream()
+            for _ in range(20):
+                got = red(d, stream=s)
+                if got != wants[k]:
+                    errors.append((k, got, wants[k]))
+        except Exception as e:      # pragma: no cover
+            errors.append((k, repr(e)))
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(4)]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    assert not errors, errors[:3]
+
+
+def test_untranslatable_functor_is_refused_when_the_object_is_made():
+    with pytest.raises(NotImplementedError, match="could not translate"):
+        cuda.Reduce(lambda a, b: int(a) + b)
+    with pytest.raises(TypeError, match="bitwise"):
+        cuda.Reduce(FC.BY_NAME["xor_and_flip"].functor)(np.zeros(4, np.float32))
+    with pytest.raises(NotImplementedError, match="dtype"):
+        cuda.Reduce(FC.BY_NAME["sum_plus_one"].functor)(np.zeros(4, np.complex64))

@@ -1,0 +1,57 @@
+"""Pins the oracle's Python restatements for general functors (oracle/cref.py
+functor_fold / functor_tree / typed_functor) against what is already pinned: the C
+restatements orc_fold_* / orc_tree_* for the four standard operators (bit for bit, with
+float32 sums, which move when the association order moves), and closed forms on wrapped
+integers for the typing."""
+
+import numpy as np
+import pytest
+
+from oracle import cref
+
+STANDARD = [("add", lambda a, b: a + b), ("mul", lambda a, b: a * b), ("max", lambda a, b: max(a, b)),
+            ("min", lambda a, b: a if a < b else b)]
+
+
+@pytest.mark.parametrize("n", [1, 2, 31, 32, 33, 127, 128, 129, 255, 1000, 8192, 8192 + 77, 8192 + 128, 20000])
+def test_tree_and_fold_orders_match_the_c_restatement(n):
+    rng = np.random.default_rng(n)
+    f32 = rng.standard_normal(n).astype(np.float32)
+    i32 = rng.integers(-2**31, 2**31, n).astype(np.int32)
+    u8 = rng.integers(0, 256, n).astype(np.uint8)
+    for name, functor in STANDARD:
+        for data, init in ((f32, 0.5), (i32, 3), (u8, 1)):
+            if name == "mul" and data.dtype.kind == "f":
+                data = (1 + data / 64).astype(np.float32)
+            assert cref.functor_tree(functor, data, init).tobytes() == cref.tree(name, data, init).tobytes()
+            assert cref.functor_fold(functor, data, init).tobytes() == cref.fold(name, data, init).tobytes()
+
+
+def test_typing_on_wrapped_integers_closed_forms():
+    rng = np.random.default_rng(5)
+    for dtype in (np.int8, np.uint8, np.int32, np.uint32, np.int64, np.uint64):
+        info = np.iinfo(dtype)
+        a = rng.integers(info.min, info.max, 3000, dtype=dtype, endpoint=True)
+        exact = [int(x) for x in a]
+        bits = 8 * np.dtype(dtype).itemsize
+
+        def wrap(v):
+            v &= (1 << bits) - 1
+            return v - (1 << bits) if info.min < 0 and v >= 1 << (bits - 1) else v
+        # a + b + 1 over n elements and init: sum + init + n
+        assert int(cref.functor_tree(lambda x, y: x + y + 1, a, 7)) == wrap(sum(exact) + 7 + len(exact))
+        # a * b + a + b = (a + 1)(b + 1) - 1
+        prod = 1
+        for x in exact + [2]:
+            prod = prod * (x + 1) % (1 << 64)
+        assert int(cref.functor_tree(lambda x, y: x * y + x + y, a, 2)) == wrap(prod - 1)
+        assert int(cref.functor_fold(lambda x, y: x * y + x + y, a, 2)) == wrap(prod - 1)
+
+
+def test_typing_of_booleans_and_float_results():
+    f = cref.typed_functor(lambda a, b: a + b, np.bool_)
+    assert f(True, True) is np.True_ and f(False, False) is np.False_
+    g = cref.typed_functor(lambda a, b: a / 2 + b / 2, np.int32)
+    assert g(np.int32(-3), np.int32(0)) == -1 and isinstance(g(1, 1), np.int32)       # towards zero
+    h = cref.typed_functor(lambda a, b: a * b, np.float32)
+    assert h(np.float32(1.1), np.float32(1.1)) == np.float32(1.1) * np.float32(1.1)
