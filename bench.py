@@ -17,6 +17,7 @@ just one of them (or copy_f32, the counter calibration kernel) as the headline.
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -132,6 +133,10 @@ def _cpu_baseline_rng(name, nthreads=4096):
             "outputs_per_s": round(nthreads * count / dt, 1), "host_cores_available": os.cpu_count()}
 
 
+def _hypot(a, b):
+    return math.sqrt(a * a + b * b)
+
+
 def _workload(name, cuda):
     """-> dict(desc, dtype, algo_bytes, units, step(i), stream, host_input, kernel)"""
     from numba_cuda_amd import random as nrandom
@@ -141,7 +146,11 @@ def _workload(name, cuda):
     mx = cuda.Reduce(lambda a, b: max(a, b))
     rng = np.random.default_rng(1)
     if name.startswith("reduce_"):
-        if name == "reduce_f32_sum" or name == "reduce_f32_max":
+        if name == "reduce_f32_functor":
+            # a functor without a kernel of its own: translated and compiled at run time
+            host = rng.standard_normal(2**28, dtype=np.float32)
+            desc = "cuda.reduce fp32 with lambda a, b: sqrt(a*a + b*b) (translated functor), 2^28 elements N(0,1), seed 1"
+        elif name == "reduce_f32_sum" or name == "reduce_f32_max":
             host = rng.standard_normal(2**28, dtype=np.float32)
             desc = "cuda.reduce fp32 %s, 2^28 elements N(0,1), seed 1" % ("sum" if name.endswith("sum") else "max")
         elif name == "reduce_f64_sum":
@@ -158,13 +167,17 @@ def _workload(name, cuda):
         res = cuda.device_array(1, dtype=host.dtype)
         red = mx if name.endswith("max") else add
         init = -np.inf if name.endswith("max") else 0
+        kernel = "reduce_kernel"
+        if name.endswith("functor"):
+            red = cuda.Reduce(_hypot)
+            kernel = "nbh_custom_reduce"
 
         def step(i):
             red(bufs[i & 1], res=res, init=init, stream=stream)
 
         return dict(desc=desc, dtype={"float32": "f32", "float64": "f64", "int64": "int64"}[host.dtype.name],
                     algo_bytes=host.nbytes, units=host.size, step=step, stream=stream, host=host,
-                    kernel="reduce_kernel", keep=(bufs, res))
+                    kernel=kernel, keep=(bufs, res))
     if name.startswith("transpose_"):
         rng = np.random.default_rng(2)
         if name == "transpose_f32":
@@ -292,15 +305,15 @@ TRAFFIC_SOURCE = {
     "rng_init": "profiles/hbm_counters_other_workloads.txt",
 }
 
-OTHER_WORKLOADS = ["reduce_f32_max", "reduce_f64_sum", "reduce_i64_sum", "transpose_f32", "transpose_f64",
+OTHER_WORKLOADS = ["reduce_f32_max", "reduce_f64_sum", "reduce_i64_sum", "reduce_f32_functor", "transpose_f32", "transpose_f64",
                    "transpose_i16", "rng_init", "rng_uniform_f32", "rng_normal_f64", "batched_reduce"]
 
 
 def _cpu_baseline(name, w, seconds):
     if name.startswith("reduce_"):
         is_max = name.endswith("max")
-        return _cpu_baseline_reduce(w["host"], target_seconds=seconds,
-                                    functor=(lambda x, y: max(x, y)) if is_max else (lambda x, y: x + y))
+        functor = _hypot if name.endswith("functor") else (lambda x, y: max(x, y)) if is_max else (lambda x, y: x + y)
+        return _cpu_baseline_reduce(w["host"], target_seconds=seconds, functor=functor)
     if name == "batched_reduce":
         return _cpu_baseline_reduce(w["host"].reshape(-1), target_seconds=seconds)
     if name.startswith("transpose_"):

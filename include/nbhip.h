@@ -218,8 +218,8 @@ int nbh_reduce_op_free(void *op);
  * association: every element and `init` enter exactly once, n applications for n
  * elements, so the result equals the reference's (kernels/reduction.py:194-265) for every
  * operation that is associative and commutative - the same condition the reference's own
- * tree imposes.  Arguments as for nbh_reduce (`scratch` is the same buffer; its ticket is
- * left alone).  Two launches on `stream`, fully asynchronous. */
+ * tree imposes.  Arguments as for nbh_reduce (`scratch` is the same buffer, used the same
+ * way: the ticket is handed back at zero).  One launch on `stream`, fully asynchronous. */
 int nbh_reduce_custom(void *op, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                       void *scratch, size_t scratch_bytes, nbh_stream_t stream);
 

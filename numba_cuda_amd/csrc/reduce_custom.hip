@@ -18,10 +18,12 @@
 // the reference's: like the reference, the result is only defined for operations that are
 // associative and commutative.
 //
-// Two launches: `nbh_custom_partials` leaves one partial (and its flag) per workgroup in
-// the scratch buffer, `nbh_custom_finish` (one workgroup) folds those, applies `init` and
-// writes `out`.  The partial slots are those of nbh_reduce's scratch buffer; the ticket in
-// its header is not touched, so one buffer serves both kinds of calls on a stream.
+// One launch of `nbh_custom_reduce`, shaped like nbh_reduce's kernel: 512-thread workgroups,
+// two per compute unit, each streaming one contiguous slice; one partial per workgroup in
+// the scratch buffer; the workgroup that draws the last ticket folds the partials, applies
+// `init` and writes `out`.  Ticket and partial slots are those of nbh_reduce's scratch
+// buffer, used the same way (the ticket is handed back at zero), so one buffer serves both
+// kinds of calls on a stream.
 #include <dlfcn.h>
 #include <hip/hiprtc.h>
 
@@ -34,11 +36,12 @@
 
 namespace {
 
-constexpr int kBlock = 256;
-constexpr int kMaxGrid = 2048;            // 8 workgroups per compute unit on a 256-CU part
-constexpr size_t kHeaderBytes = 256;      // nbh_reduce's ticket lives here
-constexpr size_t kFlagsOffset = kHeaderBytes + sizeof(uint64_t) * kMaxGrid;
-constexpr size_t kNeededBytes = kFlagsOffset + sizeof(uint32_t) * kMaxGrid;
+constexpr int kBlock = 512;               // threads per workgroup; the device source says the same
+constexpr int kUnroll = 4;
+constexpr int kGridPerCU = 2;
+constexpr int kMaxGrid = 4096;            // partial slots in nbh_reduce's scratch buffer
+constexpr size_t kHeaderBytes = 256;      // the ticket lives here
+constexpr size_t kNeededBytes = kHeaderBytes + sizeof(uint64_t) * kMaxGrid;
 constexpr int kMaxDevices = 64;
 
 // ---- the run-time compiler, loaded on first use ---------------------------------------
@@ -152,6 +155,7 @@ __device__ __forceinline__ T nbh_op(T a, T b)
 // are defined away: the translation of functors is checked that way without a device)
 
 constexpr int kItems = 16 / (int)sizeof(T);     // elements per 16-byte packet
+constexpr int kThreads = 512, kWaves = 8, kUnroll = 4;
 union nbh_packet { nbh_u32x4 raw; T item[kItems]; };
 union nbh_slot { nbh_u64 word; T value; };
 
@@ -184,8 +188,8 @@ __device__ __forceinline__ T nbh_fold_packet(const nbh_u32x4 raw)
     return v;
 }
 
-// Lane 0 of the wavefront, then thread 0 of the workgroup, ends up with every item that
-// any thread holds, each taken once.
+// Thread 0 of the workgroup ends up with every item that any thread holds, each taken
+// once, in an order that depends on nothing but the thread indices.
 __device__ __forceinline__ void nbh_fold_workgroup(T &acc, bool &have)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -196,77 +200,118 @@ __device__ __forceinline__ void nbh_fold_workgroup(T &acc, bool &have)
         if (lane + off < 64 && they_have)
             nbh_take(acc, have, nbh_value_of(theirs));
     }
-    __shared__ nbh_u64 wave_value[4];
-    __shared__ int wave_has[4];
+    __shared__ nbh_u64 wave_value[kWaves];
+    __shared__ int wave_has[kWaves];
+    __syncthreads();  // the slots may still be read from a previous fold
     if (lane == 0) {
         wave_value[wave] = nbh_word_of(acc);
         wave_has[wave] = (int)have;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        const int waves = (int)(blockDim.x + 63) >> 6;
-        for (int w = 1; w < waves; ++w)
+        for (int w = 1; w < kWaves; ++w)
             if (wave_has[w])
                 nbh_take(acc, have, nbh_value_of(wave_value[w]));
     }
 }
 
-// packets > 0: `in` is contiguous and 16-byte aligned; the first `packets` packets are read
-// whole, the fewer than kItems items after them one by one.  packets == 0: items
-// `stride` bytes apart.
-extern "C" __global__ __launch_bounds__(256) void nbh_custom_partials(const char *__restrict__ in, long long n,
-                                                                     long long stride, long long packets,
-                                                                     nbh_u64 *__restrict__ part_value,
-                                                                     unsigned *__restrict__ part_has)
+// One launch.  Every workgroup owns a contiguous, non-empty slice of the input and streams
+// it with kUnroll 16-byte non-temporal loads in flight per lane; it leaves one partial; the
+// workgroup that draws the last ticket folds the partials in index order, applies `init`
+// and writes `out`.  Partials are put in place with an agent-scope atomic exchange whose
+// result is awaited before the ticket is drawn (the protocol of nbh_reduce, for the same
+// reason: the L2 caches of the XCDs are not coherent with one another, agent-scope
+// atomics are carried out where all of them look).
+// packed != 0: items [head, head + units * kItems) are `units` aligned packets; the `head`
+// items in front and the fewer than kItems behind are taken by single lanes of workgroup 0.
+// packed == 0: `units` items, `stride` bytes apart.
+extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce(const char *__restrict__ in, long long n,
+                                                                   long long head, long long units,
+                                                                   long long stride, int packed, T init,
+                                                                   T *__restrict__ out,
+                                                                   nbh_u64 *__restrict__ partials,
+                                                                   unsigned *__restrict__ ticket)
 {
-    const long long me = blockIdx.x * 256ll + threadIdx.x, step = gridDim.x * 256ll;
+    __shared__ bool last_block;
+    const int tid = threadIdx.x;
+    const long long per = (units + gridDim.x - 1) / gridDim.x;
+    const long long begin = (long long)blockIdx.x * per;
+    long long end = begin + per;
+    if (end > units)
+        end = units;
     T acc = T();
     bool have = false;
-    if (packets > 0) {
-        const nbh_u32x4 *__restrict__ p = reinterpret_cast<const nbh_u32x4 *>(in);
-        long long k = me;
-        if (k < packets) {
-            acc = nbh_fold_packet(__builtin_nontemporal_load(p + k));
+    long long i = begin + tid;
+    if (packed) {
+        const nbh_u32x4 *__restrict__ p = reinterpret_cast<const nbh_u32x4 *>(in + head * (long long)sizeof(T));
+        if (i < end) {
+            acc = nbh_fold_packet(__builtin_nontemporal_load(p + i));
             have = true;
-            k += step;
+            i += kThreads;
         }
-        for (; k + 3 * step < packets; k += 4 * step) {
-            const nbh_u32x4 r0 = __builtin_nontemporal_load(p + k);
-            const nbh_u32x4 r1 = __builtin_nontemporal_load(p + k + step);
-            const nbh_u32x4 r2 = __builtin_nontemporal_load(p + k + 2 * step);
-            const nbh_u32x4 r3 = __builtin_nontemporal_load(p + k + 3 * step);
+        for (; i + (kUnroll - 1) * kThreads < end; i += kUnroll * kThreads) {
+            const nbh_u32x4 r0 = __builtin_nontemporal_load(p + i);
+            const nbh_u32x4 r1 = __builtin_nontemporal_load(p + i + kThreads);
+            const nbh_u32x4 r2 = __builtin_nontemporal_load(p + i + 2 * kThreads);
+            const nbh_u32x4 r3 = __builtin_nontemporal_load(p + i + 3 * kThreads);
             const T v01 = nbh_op(nbh_fold_packet(r0), nbh_fold_packet(r1));
             const T v23 = nbh_op(nbh_fold_packet(r2), nbh_fold_packet(r3));
             acc = nbh_op(acc, nbh_op(v01, v23));
         }
-        for (; k < packets; k += step)
-            acc = nbh_op(acc, nbh_fold_packet(__builtin_nontemporal_load(p + k)));
-        const long long t = packets * kItems + me;
-        if (t < n)
-            nbh_take(acc, have, reinterpret_cast<const T *>(in)[t]);
+        for (; i < end; i += kThreads)
+            acc = nbh_op(acc, nbh_fold_packet(__builtin_nontemporal_load(p + i)));
+        if (blockIdx.x == 0) {
+            const T *__restrict__ items = reinterpret_cast<const T *>(in);
+            const long long tail_begin = head + units * kItems;
+            if (tid < head)
+                nbh_take(acc, have, items[tid]);
+            else if (tail_begin + (tid - head) < n)
+                nbh_take(acc, have, items[tail_begin + (tid - head)]);
+        }
     } else {
-        for (long long i = me; i < n; i += step)
-            nbh_take(acc, have, *reinterpret_cast<const T *>(in + i * stride));
+        if (i < end) {
+            acc = *reinterpret_cast<const T *>(in + i * stride);
+            have = true;
+            i += kThreads;
+        }
+        for (; i + (kUnroll - 1) * kThreads < end; i += kUnroll * kThreads) {
+            const T v0 = *reinterpret_cast<const T *>(in + i * stride);
+            const T v1 = *reinterpret_cast<const T *>(in + (i + kThreads) * stride);
+            const T v2 = *reinterpret_cast<const T *>(in + (i + 2 * kThreads) * stride);
+            const T v3 = *reinterpret_cast<const T *>(in + (i + 3 * kThreads) * stride);
+            acc = nbh_op(acc, nbh_op(nbh_op(v0, v1), nbh_op(v2, v3)));
+        }
+        for (; i < end; i += kThreads)
+            acc = nbh_op(acc, *reinterpret_cast<const T *>(in + i * stride));
     }
-    nbh_fold_workgroup(acc, have);
-    if (threadIdx.x == 0) {
-        part_value[blockIdx.x] = nbh_word_of(acc);
-        part_has[blockIdx.x] = have ? 1u : 0u;
-    }
-}
+    nbh_fold_workgroup(acc, have);  // thread 0 has the slice's value: the slice is not empty
 
-extern "C" __global__ __launch_bounds__(256) void nbh_custom_finish(const nbh_u64 *__restrict__ part_value,
-                                                                   const unsigned *__restrict__ part_has, int count,
-                                                                   T init, T *__restrict__ out)
-{
-    T acc = T();
-    bool have = false;
-    for (int k = threadIdx.x; k < count; k += 256)
-        if (part_has[k])
-            nbh_take(acc, have, nbh_value_of(part_value[k]));
+    if (gridDim.x == 1) {
+        if (tid == 0)
+            out[0] = nbh_op(acc, init);
+        return;
+    }
+    if (tid == 0) {
+        const nbh_u64 before = __hip_atomic_exchange(&partials[blockIdx.x], nbh_word_of(acc), __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("" ::"v"(before) : "memory");  // wait until the exchange has been carried out
+        const unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_block = (t == gridDim.x - 1);
+        if (last_block)
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+    __syncthreads();
+    if (!last_block)
+        return;
+    have = false;
+    for (int k = tid; k < (int)gridDim.x; k += kThreads)
+        nbh_take(acc, have, nbh_value_of(__hip_atomic_load(&partials[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
     nbh_fold_workgroup(acc, have);
-    if (threadIdx.x == 0)
-        out[0] = have ? nbh_op(acc, init) : init;
+    if (tid == 0) {
+        out[0] = nbh_op(acc, init);
+        // leave the scratch buffer as the caller handed it over
+        __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 )NBHSRC";
 
@@ -277,7 +322,7 @@ struct CustomOp {
     std::mutex lock;
     struct Loaded {
         hipModule_t module = nullptr;
-        hipFunction_t partials = nullptr, finish = nullptr;
+        hipFunction_t reduce = nullptr;
     } on_device[kMaxDevices];
 };
 
@@ -298,20 +343,17 @@ int functions_for(CustomOp *op, CustomOp::Loaded **out)
         return (int)hipErrorInvalidDevice;
     std::lock_guard<std::mutex> hold(op->lock);
     CustomOp::Loaded &slot = op->on_device[dev];
-    if (!slot.finish) {
+    if (!slot.reduce) {
         hipModule_t m = nullptr;
         NBH_TRY(hipModuleLoadData(&m, op->code.data()));
-        hipFunction_t f1 = nullptr, f2 = nullptr;
-        hipError_t e = hipModuleGetFunction(&f1, m, "nbh_custom_partials");
-        if (e == hipSuccess)
-            e = hipModuleGetFunction(&f2, m, "nbh_custom_finish");
+        hipFunction_t f = nullptr;
+        const hipError_t e = hipModuleGetFunction(&f, m, "nbh_custom_reduce");
         if (e != hipSuccess) {
             (void)hipModuleUnload(m);
             return (int)e;
         }
         slot.module = m;
-        slot.partials = f1;
-        slot.finish = f2;
+        slot.reduce = f;
     }
     *out = &slot;
     return 0;
@@ -409,26 +451,45 @@ extern "C" int nbh_reduce_custom(void *handle, const void *in, int64_t n, int64_
     nbh_stream_report report(s);
 
     const int64_t items = 16 / (int64_t)op->elem;
-    long long packets = 0;
-    if (in_stride == (int64_t)op->elem && ((uintptr_t)in) % 16 == 0)
-        packets = n / items;
-    const int64_t threads = packets > 0 ? packets : n;
-    int64_t grid = (threads + kBlock - 1) / kBlock;
-    if (grid > kMaxGrid)
-        grid = kMaxGrid;
+    const uintptr_t addr = (uintptr_t)in;
+    if (addr % op->elem != 0 || ((uintptr_t)out) % op->elem != 0)
+        return (int)hipErrorInvalidValue;
+    const int packed = (in_stride == (int64_t)op->elem || n == 1) ? 1 : 0;
+    long long head = 0, units = n;  // units: packets when packed, items otherwise
+    if (packed) {
+        head = (long long)(((16 - (addr % 16)) % 16) / op->elem);
+        if (head > n)
+            head = n;
+        units = (n - head) / items;
+    }
+    // as many workgroups as nbh_reduce would start, then no more than have a slice each
+    const int64_t per_block = (int64_t)kBlock * kUnroll;
+    int64_t grid = (units + per_block - 1) / per_block;
+    if (grid < 32) {
+        grid = (units + kBlock - 1) / kBlock;
+        if (grid > 32)
+            grid = 32;
+    }
+    int64_t cap = (int64_t)nbh_cu_count() * kGridPerCU;
+    if (cap > kMaxGrid)
+        cap = kMaxGrid;
+    if (grid > cap)
+        grid = cap;
     if (grid < 1)
         grid = 1;
+    if (units > 0) {
+        const int64_t per = (units + grid - 1) / grid;
+        grid = (units + per - 1) / per;  // every workgroup's slice holds at least one unit
+    }
 
     const char *in_arg = static_cast<const char *>(in);
     long long n_arg = n, stride_arg = in_stride;
-    uint64_t *part_value = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kHeaderBytes);
-    unsigned *part_has = reinterpret_cast<unsigned *>(static_cast<char *>(scratch) + kFlagsOffset);
-    void *args1[] = {&in_arg, &n_arg, &stride_arg, &packets, &part_value, &part_has};
-    NBH_TRY(hipModuleLaunchKernel(fn->partials, (unsigned)grid, 1, 1, kBlock, 1, 1, 0, s, args1, nullptr));
-
-    int count = (int)grid;
+    int packed_arg = packed;
+    uint64_t *partials = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kHeaderBytes);
+    unsigned *ticket = reinterpret_cast<unsigned *>(scratch);
     // `init` travels as a kernel argument: the launch copies the element it points to
-    void *args2[] = {&part_value, &part_has, &count, const_cast<void *>(init), &out};
-    NBH_TRY(hipModuleLaunchKernel(fn->finish, 1, 1, 1, kBlock, 1, 1, 0, s, args2, nullptr));
+    void *args[] = {&in_arg, &n_arg, &head, &units, &stride_arg, &packed_arg, const_cast<void *>(init),
+                    &out, &partials, &ticket};
+    NBH_TRY(hipModuleLaunchKernel(fn->reduce, (unsigned)grid, 1, 1, kBlock, 1, 1, 0, s, args, nullptr));
     return 0;
 }

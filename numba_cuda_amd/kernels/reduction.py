@@ -9,7 +9,7 @@ the reference's JIT does), float32, float64, complex64 and complex128.
 
 Any other functor is translated (kernels/functor.py: run on recording stand-ins, typed
 with the JIT's rules, written out as C++) and compiled for the device at run time, once
-per functor and element type; nbh_reduce_custom then runs it in two launches.  Element
+per functor and element type; nbh_reduce_custom then runs it in one launch.  Element
 types there: integers, booleans and the real floating-point types.  What cannot be
 translated raises NotImplementedError - there is no host fallback.
 """
