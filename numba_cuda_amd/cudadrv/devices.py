@@ -10,32 +10,34 @@ object.
 
 import functools
 import threading
+from collections.abc import Sequence
 
 from .driver import driver
 
 
-class _DeviceList:
-    """`cuda.gpus`: indexable, iterable, `len()`-able list of devices; each entry
-    is also a context manager that makes the device current inside `with`."""
+class _DeviceList(Sequence):
+    """`cuda.gpus`: the devices as a read-only sequence (index, iterate, `len()`); each
+    entry is also a context manager that makes its device current inside `with`.  The
+    devices are asked for on first use, not at import."""
 
-    def __getattr__(self, attr):
-        if attr == "lst":
-            lst = [_DeviceContextManager(driver.get_device(i)) for i in range(driver.get_device_count())]
-            self.lst = lst
-            return lst
-        raise AttributeError(attr)
+    _entries = None
+
+    @property
+    def lst(self):
+        entries = self._entries
+        if entries is None:
+            count = driver.get_device_count()
+            entries = self._entries = [_DeviceContextManager(driver.get_device(i)) for i in range(count)]
+        return entries
 
     def __getitem__(self, devnum):
         return self.lst[devnum]
 
-    def __str__(self):
-        return ", ".join(str(d) for d in self.lst)
-
-    def __iter__(self):
-        return iter(self.lst)
-
     def __len__(self):
         return len(self.lst)
+
+    def __str__(self):
+        return ", ".join(map(str, self.lst))
 
     @property
     def current(self):
@@ -45,22 +47,28 @@ class _DeviceList:
 
 
 class _DeviceContextManager:
+    """A device that can be entered: `with cuda.gpus[i]:` selects it for the calling
+    thread and goes back to the thread's earlier device on the way out.  Everything
+    else is the device's own attribute."""
+
     def __init__(self, device):
         self._device = device
+        self._came_from = threading.local()   # per host thread: the devices to go back to
 
-    def __getattr__(self, item):
-        return getattr(self._device, item)
+    def __getattr__(self, name):
+        return getattr(self._device, name)
 
     def __enter__(self):
-        self._previous = _runtime.current_device
+        self._came_from.__dict__.setdefault("stack", []).append(_runtime.current_device)
         _runtime.get_or_create_context(self._device.id)
 
-    def __exit__(self, exc_type, exc_val, exc_tb):
-        if self._previous is not None:
-            _runtime.get_or_create_context(self._previous)
+    def __exit__(self, *exc_info):
+        earlier = self._came_from.stack.pop()
+        if earlier is not None:
+            _runtime.get_or_create_context(earlier)
 
     def __str__(self):
-        return "<Managed Device {self.id}>".format(self=self)
+        return "<Managed Device %d>" % self._device.id
 
 
 class _Runtime:
