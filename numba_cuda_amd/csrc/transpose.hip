@@ -162,10 +162,12 @@ template <> struct ShearOf<4> { using type = RingCfg<4, 256, 64, 4, 512, 1>; };
 template <> struct ShearOf<8> { using type = RingCfg<8, 128, 32, 4, 256, 1>; };
 template <> struct ShearOf<16> { using type = RingCfg<16, 64, 32, 1, 256, 1>; };
 
+constexpr int kOrderPlain = 0, kOrderByXcd = 1, kOrderPadded = 2;
+
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__restrict__ in, char *__restrict__ out,
                                                                    int64_t rows, int64_t cols, int64_t in_s0,
-                                                                   int64_t out_s0, int64_t strips_r, bool by_xcd)
+                                                                   int64_t out_s0, int64_t strips_r, int order)
 {
     constexpr int E = Cfg::E;
     using Item = typename ItemOf<E>::type;
@@ -184,13 +186,22 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
     // column bands fetch the same lines: give each XCD a contiguous share of the bands
     // so that they meet in one L2 (float32 16385^2: 4.6 -> 5.1 TB/s).
     int64_t logical = blockIdx.x;
-    if (by_xcd) {
+    if (order == kOrderByXcd) {
         const int64_t per = (int64_t)gridDim.x / 8;
         if (logical < per * 8)
             logical = (logical % 8) * per + logical / 8;
     }
-    const int64_t tile_c = logical / strips_r;
-    const int64_t strip = logical % strips_r;
+    // kOrderPadded: the strips of a column band are counted up to a multiple of 8, so that
+    // tiles side by side (same strip, neighbouring bands) run on the same XCD, strips_pad / 8
+    // dispatches apart: the line of every input row that straddles their common edge is
+    // fetched from memory once and found in that XCD's L2 the second time, while the order
+    // in which the chip walks through the matrix stays what it was.  (float64 12345 x 6789:
+    // fetched bytes 1.62 -> 1.15 x the input; the surplus workgroups leave at once.)
+    const int64_t strips_pad = order == kOrderPadded ? (strips_r + 7) / 8 * 8 : strips_r;
+    const int64_t tile_c = logical / strips_pad;
+    const int64_t strip = logical % strips_pad;
+    if (strip >= strips_r)
+        return;
     const int64_t C0 = tile_c * TC;
     const int64_t strip_begin = strip * (int64_t)(Cfg::STEPS * TR);
     int64_t strip_end = strip_begin + (int64_t)Cfg::STEPS * TR;
@@ -206,6 +217,52 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
         Item it[V];
     };
     Pack held[NP];
+
+    // Tiles of a one-step configuration that lie wholly inside the matrix, when the input
+    // rows are off the 128-byte grid too (order == kOrderPadded): nothing needs a guard, so
+    // the tile and the L rows above it arrive with ONE round of loads (the general path
+    // below waits for the L rows before it asks for the rest), and every thread then writes
+    // TR / L lines of one output row, 128 bytes apart, all read from LDS before the first
+    // store.  Measured, general path -> this one: float64 12345 x 6789 246 -> 234 us (with
+    // the padded order), float32 16100^2 391 -> 369, 12345 x 13578 259 -> 239.  With input
+    // rows ON the grid it is slower (float32 16388 x 16384 374 -> 391, float64 4099 x 20000
+    // 229 -> 243) and for 16-byte items as well (8193^2 366 -> 401): those keep the general path.
+    if constexpr (Cfg::STEPS == 1 && E < 16) {
+        if (order == kOrderPadded && strip_begin >= L && strip_begin + TR < rows && C0 + TC <= cols) {
+            constexpr int RPS = kThr / PPR;      // tile rows one round of the workgroup loads
+            constexpr int NPF = RING * PPR / kThr;
+            constexpr int NLF = TR / L;          // whole lines per output row
+            static_assert(RING * PPR % kThr == 0 && kThr % PPR == 0, "whole rounds of loads");
+            static_assert(kThr / 8 == TC && TR % L == 0, "eight lanes per output row");
+            const int64_t A = strip_begin - L;
+            const int lr0 = tid / PPR, pc = tid % PPR;
+            const char *src = in + (A + lr0) * in_s0 + (C0 + (int64_t)pc * V) * E;
+            u32x4 got[NPF];
+#pragma unroll
+            for (int k = 0; k < NPF; ++k)
+                got[k] = nbh_load16<E, false>(src + (int64_t)k * RPS * in_s0);
+#pragma unroll
+            for (int k = 0; k < NPF; ++k)  // tile row t sits in ring row t: one step, no wrap
+                *reinterpret_cast<u32x4 *>(&ring[lr0 + k * RPS][pc * V]) = got[k];
+            __syncthreads();
+            const int lc = tid >> 3, sub = tid & 7;
+            char *row = out + (C0 + lc) * out_s0;
+            const int phase = (int)(((uintptr_t)row % 128) / E);
+            const int64_t lo = strip_begin - (phase + strip_begin) % L;  // in (strip_begin - L, strip_begin]
+            const int d = (int)(lo - A) + sub * V;                         // tile row of this lane's first item
+            Pack p[NLF];
+#pragma unroll
+            for (int i = 0; i < NLF; ++i)
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    p[i].it[j] = ring[d + i * L + j][lc];
+            char *dst = row + (lo + sub * V) * E;  // 16-byte aligned: lo starts a line
+#pragma unroll
+            for (int i = 0; i < NLF; ++i)
+                __builtin_nontemporal_store(p[i].pk, reinterpret_cast<u32x4 *>(dst + i * 128));
+            return;
+        }
+    }
 
     auto fetch = [&](int64_t from, int64_t to) {  // rows [from, to) -> held
         const int count = (int)(to - from) * PPR;
@@ -430,13 +487,18 @@ int launch_sheared_cfg(const void *in, void *out, int64_t rows, int64_t cols, in
     constexpr int TR = Cfg::RING - 128 / E;
     const int64_t strips_r = (rows + (int64_t)Cfg::STEPS * TR - 1) / ((int64_t)Cfg::STEPS * TR);
     const int64_t tiles_c = (cols + Cfg::TC - 1) / Cfg::TC;
-    const int64_t blocks = strips_r * tiles_c;
+    const bool ragged_in = (((uint64_t)(uintptr_t)in | (uint64_t)in_s0) % 128) != 0;
+    int order = kOrderPlain;
+    if (ragged_in && Cfg::TC * E <= 128)
+        order = kOrderByXcd;
+    else if (ragged_in && Cfg::STEPS == 1 && E < 16)
+        order = kOrderPadded;
+    const int64_t strips_grid = order == kOrderPadded ? (strips_r + 7) / 8 * 8 : strips_r;
+    const int64_t blocks = strips_grid * tiles_c;
     if (blocks > 0x7fffffffLL)
         return (int)hipErrorInvalidValue;
-    const bool ragged_in = (((uint64_t)(uintptr_t)in | (uint64_t)in_s0) % 128) != 0;
-    const bool by_xcd = ragged_in && Cfg::TC * E <= 128;
     hipLaunchKernelGGL((transpose_sheared<Cfg>), dim3((unsigned)blocks), dim3(Cfg::THREADS), 0, stream,
-                       (const char *)in, (char *)out, rows, cols, in_s0, out_s0, strips_r, by_xcd);
+                       (const char *)in, (char *)out, rows, cols, in_s0, out_s0, strips_r, order);
     return nbh_launch_status();
 }
 

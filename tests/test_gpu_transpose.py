@@ -140,6 +140,25 @@ def test_row_padded_inputs_and_outputs():
     np.testing.assert_array_equal(dst_full.copy_to_host(), want)
 
 
+@pytest.mark.parametrize("dtype", [np.int16, np.uint32, np.float64, np.complex128])
+@pytest.mark.parametrize("shape", [(1237, 1093), (3001, 2777)])
+def test_ragged_views_with_interior_and_edge_tiles(shape, dtype):
+    """Both sides off the 128-byte grid (pitched rows, item-aligned bases): large enough that
+    the ring kernel runs tiles wholly inside the matrix as well as every kind of edge tile."""
+    dtype = np.dtype(dtype)
+    rows, cols = shape
+    _say("transpose ragged views", shape, dtype)
+    rng = np.random.default_rng(rows + cols + dtype.itemsize)
+    big = rng.integers(0, 256, (rows, (cols + 3) * dtype.itemsize), dtype=np.uint8).view(dtype)
+    src = cuda.to_device(big)[:, 1:1 + cols]
+    dst_full = cuda.to_device(np.full((cols, rows + 5), 0, dtype=np.uint8).astype(dtype))
+    dst = dst_full[:, 2:2 + rows]
+    transpose(src, dst)
+    want = np.zeros((cols, rows + 5), dtype)
+    want[:, 2:2 + rows] = big[:, 1:1 + cols].T
+    assert _same_bytes(dst_full.copy_to_host(), want)
+
+
 # ---- full-size matrices, seed 2 --------- ------------------------------------------------
 
 def test_fullsize_float32_16384_square():
