@@ -156,8 +156,10 @@ template <int E_, int RING_, int TC_, int PAD_, int THREADS_, int STEPS_> struct
 // runs of every output row are written by one workgroup at one time) and so do short
 // strips: with one step per workgroup there are more, shorter workgroups in flight and
 // the L rows above a strip, read a second time, cost less than the lost overlap did.
+// 2-byte items: 256 x 64 in two steps with 256 threads -> one step of 192 rows with 512
+// threads and the unguarded interior path: 8193 x 32769 214 -> 206 us, 30001 x 7001 195 -> 183.
 template <int E> struct ShearOf;
-template <> struct ShearOf<2> { using type = RingCfg<2, 256, 64, 2, 256, 2>; };
+template <> struct ShearOf<2> { using type = RingCfg<2, 256, 64, 8, 512, 1>; };
 template <> struct ShearOf<4> { using type = RingCfg<4, 256, 64, 4, 512, 1>; };
 template <> struct ShearOf<8> { using type = RingCfg<8, 128, 32, 4, 256, 1>; };
 template <> struct ShearOf<16> { using type = RingCfg<16, 64, 32, 1, 256, 1>; };
@@ -167,7 +169,7 @@ constexpr int kOrderPlain = 0, kOrderByXcd = 1, kOrderPadded = 2;
 template <typename Cfg>
 __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__restrict__ in, char *__restrict__ out,
                                                                    int64_t rows, int64_t cols, int64_t in_s0,
-                                                                   int64_t out_s0, int64_t strips_r, int order)
+                                                                   int64_t out_s0, int64_t strips_r, int order, bool lean)
 {
     constexpr int E = Cfg::E;
     using Item = typename ItemOf<E>::type;
@@ -218,17 +220,19 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
     };
     Pack held[NP];
 
-    // Tiles of a one-step configuration that lie wholly inside the matrix, when the input
-    // rows are off the 128-byte grid too (order == kOrderPadded): nothing needs a guard, so
+    // Tiles of a one-step configuration that lie wholly inside the matrix (`lean`: the host
+    // asks for this path where it was measured to win): nothing needs a guard, so
     // the tile and the L rows above it arrive with ONE round of loads (the general path
     // below waits for the L rows before it asks for the rest), and every thread then writes
     // TR / L lines of one output row, 128 bytes apart, all read from LDS before the first
     // store.  Measured, general path -> this one: float64 12345 x 6789 246 -> 234 us (with
     // the padded order), float32 16100^2 391 -> 369, 12345 x 13578 259 -> 239.  With input
-    // rows ON the grid it is slower (float32 16388 x 16384 374 -> 391, float64 4099 x 20000
-    // 229 -> 243) and for 16-byte items as well (8193^2 366 -> 401): those keep the general path.
+    // rows ON the grid it is slower for 4- and 8-byte items (float32 16388 x 16384 374 -> 391,
+    // float64 4099 x 20000 229 -> 243) and for 16-byte items always (8193^2 366 -> 401):
+    // those keep the general path.  2-byte items gain either way (8193 x 32769 214 -> 206,
+    // 10001 x 12001 88 -> 75, input rows on the grid 8193 x 32768 206 -> 205).
     if constexpr (Cfg::STEPS == 1 && E < 16) {
-        if (order == kOrderPadded && strip_begin >= L && strip_begin + TR < rows && C0 + TC <= cols) {
+        if (lean && strip_begin >= L && strip_begin + TR < rows && C0 + TC <= cols) {
             constexpr int RPS = kThr / PPR;      // tile rows one round of the workgroup loads
             constexpr int NPF = RING * PPR / kThr;
             constexpr int NLF = TR / L;          // whole lines per output row
@@ -497,8 +501,9 @@ int launch_sheared_cfg(const void *in, void *out, int64_t rows, int64_t cols, in
     const int64_t blocks = strips_grid * tiles_c;
     if (blocks > 0x7fffffffLL)
         return (int)hipErrorInvalidValue;
+    const bool lean = Cfg::STEPS == 1 && (E == 2 || (order == kOrderPadded && E < 16));
     hipLaunchKernelGGL((transpose_sheared<Cfg>), dim3((unsigned)blocks), dim3(Cfg::THREADS), 0, stream,
-                       (const char *)in, (char *)out, rows, cols, in_s0, out_s0, strips_r, order);
+                       (const char *)in, (char *)out, rows, cols, in_s0, out_s0, strips_r, order, lean);
     return nbh_launch_status();
 }
 
