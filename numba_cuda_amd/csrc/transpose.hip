@@ -14,8 +14,14 @@
 //               Measured on MI355X (float32 16384^2): square 64x64 tiles in
 //               column-fastest order 4.5 TB/s whether staged through LDS or
 //               registers; row-fastest order 5.4 TB/s; 256 x 64 tiles with
-//               non-temporal loads and stores 6.0 TB/s.  A tile that tall would
-//               need 64 KiB of LDS per workgroup; in registers it needs none.
+//               non-temporal loads and stores 6.0 TB/s; 256 x 32 tiles with at most
+//               three workgroups per compute unit 6.1 TB/s.  A tile that tall would
+//               need tens of KiB of LDS per workgroup; in registers it needs none.
+//               Where the time goes (float32 16384^2, 256 x 32 tiles): the loads alone
+//               take 156 us, the stores alone 168 us, both patterns issued side by
+//               side 360 us whether or not the stores depend on the loads - reads and
+//               writes mixed cost this memory more than their sum unless both streams
+//               are perfectly linear (a flat copy of the same bytes: 320 us).
 //               Non-temporal access only pays when every row starts on a 128-byte
 //               line (16384-wide float32: 6.0 vs 5.4 TB/s); when rows straddle
 //               lines it is far worse than cached access (16388-wide: 2.3 vs
@@ -55,7 +61,7 @@ typedef nbh_u32x4 u32x4;
 template <int E> struct ShapeOf;
 template <> struct ShapeOf<1> { static constexpr int WR = 4, WC = 1, REP = 1; };   // 512 x 128
 template <> struct ShapeOf<2> { static constexpr int WR = 4, WC = 1, REP = 1; };   // 256 x 64
-template <> struct ShapeOf<4> { static constexpr int WR = 2, WC = 2, REP = 4; };   // 256 x 64
+template <> struct ShapeOf<4> { static constexpr int WR = 4, WC = 1, REP = 2; };   // 256 x 32
 template <> struct ShapeOf<8> { static constexpr int WR = 2, WC = 2, REP = 4; };   // 128 x 32
 template <> struct ShapeOf<16> { static constexpr int WR = 2, WC = 2, REP = 4; };  //  64 x 16
 
@@ -474,12 +480,23 @@ int launch_packets(const void *in, void *out, int64_t rows, int64_t cols, int64_
     // stream past the caches only if every row of both arrays starts on a 128-byte line
     const uint64_t mix = (uint64_t)(uintptr_t)in | (uint64_t)(uintptr_t)out | (uint64_t)in_s0 | (uint64_t)out_s0;
     const dim3 grid((unsigned)tiles), block(64 * Shape::WR * Shape::WC);
+    // Large matrices run with fewer workgroups per compute unit than would fit: what the chip
+    // has in flight then covers a narrower window of both matrices, which the memory takes
+    // better.  The kernel uses no LDS; asking for a third of a compute unit's LDS per
+    // workgroup is the throttle (at most three workgroups per compute unit).  Measured, us,
+    // free -> throttled: float32 16384^2 365 -> 353, 16000^2 363 -> 348, 8192 x 32768 372 ->
+    // 358; float64 8192 x 16384 355 -> 345, 4096 x 32768 357 -> 340; int16 32768^2 766 -> 720,
+    // 20000 x 20032 369 -> 347.  Below the thresholds it loses (float32 8192^2 96 -> 107,
+    // float64 8192^2 186 -> 195); 1- and 16-byte items never gain.
+    const double moved = 2.0 * (double)rows * (double)cols * E;
+    const double threshold = E == 4 ? 0.75 * (1u << 30) : 1.5 * (1u << 30);
+    const unsigned throttle = ((E == 2 || E == 4 || E == 8) && moved >= threshold) ? 54000u : 0u;
     if (mix % 128 == 0)
-        hipLaunchKernelGGL((transpose_packets<E, true, Shape>), grid, block, 0, stream, (const char *)in, (char *)out,
-                           rows, cols, in_s0, out_s0, tiles_r);
+        hipLaunchKernelGGL((transpose_packets<E, true, Shape>), grid, block, throttle, stream, (const char *)in,
+                           (char *)out, rows, cols, in_s0, out_s0, tiles_r);
     else
-        hipLaunchKernelGGL((transpose_packets<E, false, Shape>), grid, block, 0, stream, (const char *)in, (char *)out,
-                           rows, cols, in_s0, out_s0, tiles_r);
+        hipLaunchKernelGGL((transpose_packets<E, false, Shape>), grid, block, throttle, stream, (const char *)in,
+                           (char *)out, rows, cols, in_s0, out_s0, tiles_r);
     return nbh_launch_status();
 }
 
