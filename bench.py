@@ -37,17 +37,17 @@ MEASURED_TRAFFIC = {
     "reduce_f32_sum": 1073810755,
     # profiles/copy_flat_f32_2p28.txt: the calibration kernel itself
     "copy_f32": 2147483648,
-    # profiles/transpose_packets_f32_16384sq.txt: 1 073 772 464 B fetched + 1 073 962 931 B written
-    "transpose_f32": 2147735395,
+    # profiles/transpose_packets_f32_16384sq.txt: 1 073 761 075 B fetched + 1 074 512 910 B written
+    "transpose_f32": 2148273985,
     # profiles/xoroshiro_fill_and_init_2p24.txt: 268 618 773 B fetched + 4 563 547 721 B written
     "rng_uniform_f32": 4832166494,
-    # profiles/transpose_sheared_f64_12345x6789.txt: 1 083 619 701 B fetched + 670 476 024 B written
-    "transpose_f64": 1754095725,
+    # profiles/transpose_sheared_f64_12345x6789.txt: 768 287 439 B fetched + 670 489 125 B written
+    "transpose_f64": 1438776564,
     # profiles/hbm_counters_other_workloads.txt
     "reduce_f32_max": 1073822046,
     "reduce_f64_sum": 1073820062,
     "reduce_i64_sum": 2147534810,
-    "transpose_i16": 1073845912,
+    "transpose_i16": 1073901040,      # profiles/transpose_packets_f32_16384sq.txt, last section
     "rng_normal_f64": 2684437180,
     "rng_init": 269594109,
 }
@@ -300,7 +300,7 @@ TRAFFIC_SOURCE = {
     "reduce_f32_max": "profiles/hbm_counters_other_workloads.txt",
     "reduce_f64_sum": "profiles/hbm_counters_other_workloads.txt",
     "reduce_i64_sum": "profiles/hbm_counters_other_workloads.txt",
-    "transpose_i16": "profiles/hbm_counters_other_workloads.txt",
+    "transpose_i16": "profiles/transpose_packets_f32_16384sq.txt",
     "rng_normal_f64": "profiles/hbm_counters_other_workloads.txt",
     "rng_init": "profiles/hbm_counters_other_workloads.txt",
 }
