@@ -27,7 +27,7 @@ from numba_cuda_amd.api import (_contiguous_strides_like_array, _order_like_arra
                                 current_context, gpus, require_context)
 from numba_cuda_amd.args import In, InOut, Out  # noqa: F401
 from numba_cuda_amd import kernels  # noqa: F401
-from numba_cuda_amd.kernels import reduction as _reduction
+from numba_cuda_amd.kernels import reduction  # noqa: F401  (the reference exposes the module as cuda.reduction)
 from numba_cuda_amd.kernels import transpose as _transpose  # noqa: F401
 from numba_cuda_amd.kernels.reduction import Reduce
 from numba_cuda_amd import random  # noqa: F401

@@ -314,3 +314,8 @@ def is_float16_supported():
 
 def is_bfloat16_supported():
     return True
+
+
+def is_fp8_supported():
+    "gfx950 has 8-bit floating-point conversions and matrix instructions (reference: api.py:108-113)."
+    return True

@@ -238,6 +238,21 @@ class Device:
         if self.primary_context is not None:
             self.primary_context.reset()
 
+    def release_primary_context(self):
+        """Forget this device's context object after releasing what it holds (reference
+        :559-565).  HIP keeps its own implicit context per device; the next use builds a
+        fresh bookkeeping object."""
+        with self._ctx_lock:
+            ctx, self.primary_context = self.primary_context, None
+        if ctx is not None:
+            ctx.reset()
+
+    # What the element types need from the hardware (reference :576-586 asks the compute
+    # capability): every device this library runs on converts and computes in these.
+    supports_float16 = True
+    supports_bfloat16 = True
+    supports_fp8 = True
+
     def __repr__(self):
         return "<HIP device %d '%s'>" % (self.id, self.name)
 
