@@ -39,6 +39,20 @@ HOSTBUF_SRC = os.path.join(PKG_DIR, "cext", "hostbuf.c")
 HOSTBUF_PATH = os.path.join(PKG_DIR, "_hostbuf" + sysconfig.get_config_var("EXT_SUFFIX"))
 
 
+def hostbuf_needs_building():
+    """True when the extension module is missing or older than cext/hostbuf.c (a module that
+    is already imported cannot be replaced, so this is asked before the first import)."""
+    source = os.path.join(PKG_DIR, "cext", "hostbuf.c")
+    try:
+        built = os.stat(HOSTBUF_PATH).st_mtime
+    except OSError:
+        return True
+    try:
+        return os.stat(source).st_mtime > built
+    except OSError:
+        return False                     # no source beside it: what is built is what there is
+
+
 def build_hostbuf(verbose=False):
     """Compile cext/hostbuf.c into the extension module numba_cuda_amd._hostbuf."""
     cc = os.environ.get("CC") or shutil.which("gcc") or shutil.which("cc")

@@ -10,6 +10,8 @@
  *   extents(obj)            half-open byte range [lo, hi) its items occupy, strides of
  *                           either sign, empty when any extent is zero
  *   extents_of(shape, strides, itemsize)  the same from a description, relative to 0
+ *   reduce_into(codes, arr, res, init, stream, ...)  Reduce.__call__ with `res=` for the plain
+ *                           case, from the array objects to the launch (described at the function)
  *   call_reduce(entry, op, dtype, in, n, stride, init, out, scratch, scratch_bytes, stream)
  *                           calls the library's nbh_reduce through its address, all
  *                           arguments plain integers: the launch path of Reduce.__call__
@@ -216,7 +218,119 @@ static PyObject *hb_call_reduce(PyObject *mod, PyObject *const *args, Py_ssize_t
     return PyLong_FromLong(status);
 }
 
+/* reduce_into(codes, arr, res, init, stream, thread_state, stream_type, init_cache, lib)
+ *
+ * The whole of Reduce.__call__(arr, res=res, init=init, stream=stream) for the plain case, so
+ * that a small reduction costs the host little more than the launch itself: both arrays carry
+ * a cached description `_rk` = (address, items, stride in bytes, dtype) that the Python path
+ * stores on its first visit, `codes` maps the dtype to (operator code, element code), the
+ * calling thread's context holds the scratch buffer per stream handle, `init_cache` maps
+ * (dtype, int) to the address of the converted initial value, `lib` is the loaded library
+ * object with the address of nbh_reduce in `_reduce_entry`.  Anything out of the ordinary -
+ * no description yet, dtypes that are not the same object, an empty array, a stream that is
+ * not a Stream of ours, the per-thread default stream, no scratch buffer yet, an initial value
+ * that is not a cached int - returns NotImplemented and the Python path does the call (and
+ * raises what there is to raise).  Returns None after a launch, or the error status as int. */
+static PyObject *str_rk, *str_handle, *str_ctx, *str_prepared, *str_scratch, *str_entry;
+
+static PyObject *hb_reduce_into(PyObject *mod, PyObject *const *args, Py_ssize_t nargs)
+{
+    if (nargs != 9) {
+        PyErr_SetString(PyExc_TypeError, "reduce_into takes 9 arguments");
+        return NULL;
+    }
+    PyObject *codes = args[0], *arr = args[1], *res = args[2], *init = args[3], *stream = args[4];
+    PyObject *tls = args[5], *stream_type = args[6], *init_cache = args[7];
+    PyObject *rk = NULL, *rr = NULL, *handle = NULL, *ctx = NULL, *flag = NULL, *table = NULL, *key = NULL;
+    PyObject *entry_obj = NULL;
+    PyObject *result = NULL;  /* NULL at `out` without an exception set: NotImplemented */
+
+    if (!PyDict_CheckExact(codes) || !PyDict_CheckExact(init_cache) || !PyLong_CheckExact(init) ||
+        (PyObject *)Py_TYPE(stream) != stream_type)
+        goto out;
+    rk = PyObject_GetAttr(arr, str_rk);
+    if (!rk)
+        goto out;
+    rr = PyObject_GetAttr(res, str_rk);
+    if (!rr)
+        goto out;
+    if (!PyTuple_CheckExact(rk) || PyTuple_GET_SIZE(rk) != 4 || !PyTuple_CheckExact(rr) || PyTuple_GET_SIZE(rr) != 4)
+        goto out;
+    PyObject *dtype = PyTuple_GET_ITEM(rk, 3);
+    if (PyTuple_GET_ITEM(rr, 3) != dtype)
+        goto out;
+    PyObject *pair = PyDict_GetItemWithError(codes, dtype);  /* borrowed */
+    if (!pair || !PyTuple_CheckExact(pair) || PyTuple_GET_SIZE(pair) != 2)
+        goto out;
+    handle = PyObject_GetAttr(stream, str_handle);
+    if (!handle || !PyLong_CheckExact(handle))
+        goto out;
+    ctx = PyObject_GetAttr(tls, str_ctx);
+    if (!ctx || ctx == Py_None)
+        goto out;
+    flag = PyObject_GetAttr(ctx, str_prepared);
+    if (flag != Py_True)
+        goto out;
+    table = PyObject_GetAttr(ctx, str_scratch);
+    if (!table || !PyDict_CheckExact(table))
+        goto out;
+    PyObject *scratch = PyDict_GetItemWithError(table, handle);  /* borrowed */
+    if (!scratch || !PyTuple_CheckExact(scratch) || PyTuple_GET_SIZE(scratch) < 2)
+        goto out;
+    key = PyTuple_Pack(2, dtype, init);
+    if (!key)
+        goto out;
+    PyObject *init_addr = PyDict_GetItemWithError(init_cache, key);  /* borrowed */
+    if (!init_addr)
+        goto out;
+    {
+        unsigned long long entry, in, init_ptr, dst, scr, scr_bytes, hstream;
+        entry_obj = PyObject_GetAttr(args[8], str_entry);
+        if (!entry_obj)
+            goto out;
+        if (as_word(entry_obj, &entry) || as_word(PyTuple_GET_ITEM(rk, 0), &in) || as_word(init_addr, &init_ptr) ||
+            as_word(PyTuple_GET_ITEM(rr, 0), &dst) || as_word(PyTuple_GET_ITEM(scratch, 0), &scr) ||
+            as_word(PyTuple_GET_ITEM(scratch, 1), &scr_bytes) || as_word(handle, &hstream))
+            goto out;
+        const long op = PyLong_AsLong(PyTuple_GET_ITEM(pair, 0)), code = PyLong_AsLong(PyTuple_GET_ITEM(pair, 1));
+        const long long n = PyLong_AsLongLong(PyTuple_GET_ITEM(rk, 1));
+        const long long stride = PyLong_AsLongLong(PyTuple_GET_ITEM(rk, 2));
+        const long long room = PyLong_AsLongLong(PyTuple_GET_ITEM(rr, 1));
+        /* the per-thread default stream keeps its scratch per host thread: Python's business */
+        if (PyErr_Occurred() || !entry || n < 1 || room < 1 || hstream == 2)
+            goto out;
+        int status;
+        Py_BEGIN_ALLOW_THREADS
+        status = ((nbh_reduce_fn)(uintptr_t)entry)((int)op, (int)code, (const void *)(uintptr_t)in, (int64_t)n,
+                                                   (int64_t)stride, (const void *)(uintptr_t)init_ptr,
+                                                   (void *)(uintptr_t)dst, (void *)(uintptr_t)scr, (size_t)scr_bytes,
+                                                   (void *)(uintptr_t)hstream);
+        Py_END_ALLOW_THREADS
+        if (status == 0) {
+            result = Py_None;
+            Py_INCREF(result);
+        } else {
+            result = PyLong_FromLong(status);
+        }
+    }
+out:
+    Py_XDECREF(rk);
+    Py_XDECREF(rr);
+    Py_XDECREF(handle);
+    Py_XDECREF(ctx);
+    Py_XDECREF(flag);
+    Py_XDECREF(table);
+    Py_XDECREF(key);
+    Py_XDECREF(entry_obj);
+    if (result)
+        return result;
+    PyErr_Clear();  /* a missing attribute or the like: the Python path will say what is wrong */
+    Py_RETURN_NOTIMPLEMENTED;
+}
+
 static PyMethodDef hb_methods[] = {
+    {"reduce_into", (PyCFunction)(void (*)(void))hb_reduce_into, METH_FASTCALL,
+     "reduce_into(codes, arr, res, init, stream, thread_state, stream_type, init_cache, lib) -> None | status | NotImplemented"},
     {"call_reduce", (PyCFunction)(void (*)(void))hb_call_reduce, METH_FASTCALL,
      "call_reduce(entry, op, dtype, in, n, stride, init, out, scratch, scratch_bytes, stream) -> status"},
     {"address", hb_address, METH_VARARGS, "address(obj, writable=True) -> int"},
@@ -236,6 +350,16 @@ PyMODINIT_FUNC PyInit__hostbuf(void)
     PyObject *m = PyModule_Create(&hb_module);
     if (!m)
         return NULL;
+    str_rk = PyUnicode_InternFromString("_rk");
+    str_handle = PyUnicode_InternFromString("handle");
+    str_ctx = PyUnicode_InternFromString("ctx");
+    str_prepared = PyUnicode_InternFromString("prepared");
+    str_scratch = PyUnicode_InternFromString("_scratch");
+    str_entry = PyUnicode_InternFromString("_reduce_entry");
+    if (!str_rk || !str_handle || !str_ctx || !str_prepared || !str_scratch || !str_entry) {
+        Py_DECREF(m);
+        return NULL;
+    }
     Py_INCREF(&HostBufferType);
     if (PyModule_AddObject(m, "HostBuffer", (PyObject *)&HostBufferType) < 0) {
         Py_DECREF(&HostBufferType);

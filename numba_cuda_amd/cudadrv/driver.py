@@ -30,12 +30,11 @@ import numpy as np
 
 from numba_cuda_amd import _lib
 
-try:
-    from numba_cuda_amd import _hostbuf
-except ImportError:                      # not built yet: one gcc call, about a second
-    from numba_cuda_amd import _build
+from numba_cuda_amd import _build
+
+if _build.hostbuf_needs_building():      # not built yet, or older than its source: one gcc call, about a second
     _build.build_hostbuf()
-    from numba_cuda_amd import _hostbuf
+from numba_cuda_amd import _hostbuf
 from numba_cuda_amd.core import config
 from numba_cuda_amd.core.errors import CudaDriverError, CudaSupportError  # noqa: F401
 

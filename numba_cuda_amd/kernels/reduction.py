@@ -237,7 +237,18 @@ class Reduce:
         Returns the result as a NumPy scalar, or None when `res` is given.
         """
         # This is the whole per-call cost of small reductions (a 256 KiB row takes the
-        # device 3 us): plain attribute reads, dictionary look-ups and one native call.
+        # device 3 us).  The plain case with `res=` goes from the array objects to the
+        # launch in native code (arrays this path has seen before carry their address,
+        # length, stride and dtype as `_rk`); everything else, and whatever that call
+        # declines, takes the path below: plain attribute reads, dictionary look-ups and
+        # one native call.
+        if res is not None and size is None and not self._custom:
+            rc = _reduce_into(self._codes, arr, res, init, stream, _thread_state, _Stream, _INT_INIT,
+                              _driver.driver.lib)
+            if rc is None:
+                return None
+            if rc is not NotImplemented:
+                _driver.driver.check("nbh_reduce", rc)
         if arr.ndim != 1:
             raise TypeError("only support 1D array")
         if size is not None:
@@ -285,6 +296,14 @@ class Reduce:
             except AttributeError:
                 out_ptr = res.device_ctypes_pointer.value
             if entry:
+                if size is None:
+                    # what the native passage needs to know about the two arrays next time
+                    try:
+                        arr._rk = (in_ptr, n, arr.strides[0], dtype)
+                        if res.ndim == 1 and res.size >= 1:
+                            res._rk = (out_ptr, res.size, res.strides[0], res.dtype)
+                    except AttributeError:
+                        pass
                 rc = _call_reduce(entry, codes[0], codes[1], in_ptr, n, arr.strides[0], init_ptr, out_ptr,
                                   scratch[0], scratch[1], hstream)
             else:
@@ -372,6 +391,7 @@ _Stream = _driver.Stream
 _PER_THREAD = _driver.HIP_STREAM_PER_THREAD
 _thread_state = devices._runtime._tls
 _call_reduce = _driver._hostbuf.call_reduce
+_reduce_into = _driver._hostbuf.reduce_into
 
 def _entry_address(lib):
     """Address of the library's nbh_reduce for call_reduce, kept on the library object
