@@ -159,6 +159,29 @@ def test_ragged_views_with_interior_and_edge_tiles(shape, dtype):
     assert _same_bytes(dst_full.copy_to_host(), want)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_pitches_and_offsets(seed):
+    """Shapes, row pitches and base offsets drawn at random, every packet size: tiles inside
+    the matrix, on every edge, and the empty workgroups of a padded grid all occur."""
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(14):
+        itemsize = int(rng.choice([1, 2, 4, 8, 16]))
+        dtype = np.dtype({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64, 16: np.complex128}[itemsize])
+        rows = int(rng.integers(1, 2600))
+        cols = int(rng.integers(1, 2600))
+        pad_in, pad_out = int(rng.integers(0, 40)), int(rng.integers(0, 40))
+        off_in, off_out = int(rng.integers(0, pad_in + 1)), int(rng.integers(0, pad_out + 1))
+        _say("transpose random", seed, case, dtype, (rows, cols), (pad_in, off_in), (pad_out, off_out))
+        big = rng.integers(0, 256, (rows, (cols + pad_in) * itemsize), dtype=np.uint8).view(dtype)
+        src = cuda.to_device(big)[:, off_in:off_in + cols]
+        dst_full = cuda.to_device(np.zeros((cols, rows + pad_out), dtype))
+        dst = dst_full[:, off_out:off_out + rows]
+        transpose(src, dst)
+        want = np.zeros((cols, rows + pad_out), dtype)
+        want[:, off_out:off_out + rows] = big[:, off_in:off_in + cols].T
+        assert _same_bytes(dst_full.copy_to_host(), want), (dtype, rows, cols, pad_in, off_in, pad_out, off_out)
+
+
 # ---- full-size matrices, seed 2 --------- ------------------------------------------------
 
 def test_fullsize_float32_16384_square():
