@@ -173,6 +173,17 @@ size_t nbh_reduce_scratch_bytes(void);
 int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                void *scratch, size_t scratch_bytes, nbh_stream_t stream);
 
+/* The same reduction with the reference's association, operation for operation:
+ * kernels/reduction.py:194-265 Reduce.__call__ launching gpu_reduce_block_strided (:143-166:
+ * device_reduce_full_block :43-97, inner_warp_reduction :22-41, device_reduce_partial_block
+ * :99-141) over the full blocks, the remainder and the partials.  For float16, float32,
+ * float64 and the complex types the result has the bits a run of the reference's kernels
+ * produces (sums and products round in the same places; max / min treat NaN and signed zeros
+ * alike); integers and booleans go to nbh_reduce, whose result is the same in any order.
+ * Arguments, scratch buffer and asynchrony as for nbh_reduce; one launch. */
+int nbh_reduce_ordered(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
+                       void *scratch, size_t scratch_bytes, nbh_stream_t stream);
+
 /* nbh_reduce for callers that cannot allocate device memory: code under stream (graph)
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
  * in the reference (whose Reduce.__call__ allocates its partials on every call,

@@ -35,6 +35,9 @@ def reload_config():
     g["CUDA_LOW_OCCUPANCY_WARNINGS"] = _readenv("NUMBA_CUDA_LOW_OCCUPANCY_WARNINGS", int, 1)
     g["CUDA_ARRAY_INTERFACE_SYNC"] = _readenv("NUMBA_CUDA_ARRAY_INTERFACE_SYNC", int, 1)
     g["CUDA_MEMORY_MANAGER"] = _readenv("NUMBA_CUDA_MEMORY_MANAGER", str, "default")
+    # not in the reference: 1 makes Reduce apply its operator in the association order of the
+    # reference's kernels, so that floating-point results have the reference's bits
+    g["CUDA_REDUCE_REFERENCE_ORDER"] = _readenv("NUMBA_CUDA_REDUCE_REFERENCE_ORDER", int, 0)
 
 
 reload_config()

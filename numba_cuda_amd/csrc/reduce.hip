@@ -394,6 +394,378 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
     }
 }
 
+// ---- the reference's order of association ------------------------------------------------
+// nbh_reduce_ordered: the same reduction with every operation applied to the same pair of
+// values, in the same order, as a run of the reference's kernels (kernels/reduction.py:22-166
+// launched as in :233-258), so that floating-point results come out bit for bit - sums,
+// products, and what max / min make of NaN and signed zeros.
+//
+// The reference's order: with F = n rounded down to a multiple of 128 and G = min(F / 128, 64)
+// blocks of 128 threads, thread g < S = 128 G folds a[g], a[g + S], a[g + 2 S], ... below F
+// from left to right (:70-78); each warp of 32 runs the tree (l, l+16), (l, l+8) ... (l, l+1)
+// (:22-41); a block is (w0 op w2) op (w1 op w3) (:88-97); block 0 takes `init` in (:163-164);
+// the n - F values behind go through the one-block routine (:99-141: a full warp is a tree,
+// the last warp a left fold, the warps a left fold) and so do the partials (:256-258).
+//
+// At most 8192 chains, each strictly sequential - but every 32 consecutive chains read one
+// contiguous piece of 32 items from every "row" of S items, so a workgroup owns one of the
+// reference's warps: eight wavefronts load rows of that piece, 16 bytes per lane, two batches
+// of eight rounds in flight, and park them in LDS; 32 lanes of a ninth wavefront do nothing
+// but add down the parked rows, one chain each - 512 dependent operations per 64 KiB batch,
+// about as long as the memory takes to deliver the next one.  One launch: warp results
+// are published like the partials of reduce_kernel, the workgroup that draws the last
+// ticket does the small rest the way the reference's kernels do.
+constexpr int kOrdLoaders = 512;                 // lanes that load and park
+constexpr int kOrdThreads = kOrdLoaders + 64;    // and one more wavefront that runs the chains
+constexpr int kOrdRounds = 8;      // 16-byte loads in flight per lane
+constexpr int kRefWarp = 32, kRefBlock = 128, kRefMaxGrid = 64;
+
+// value of lane `lane + delta` (wave64 lanes; delta < 32)
+template <typename A> __device__ __forceinline__ A lane_below(A v, int delta)
+{
+    constexpr int kDwords = (int)((sizeof(A) + 3) / 4);
+    union {
+        A a;
+        uint32_t w[kDwords];
+    } u;
+    u.w[kDwords - 1] = 0;
+    u.a = v;
+#pragma unroll
+    for (int k = 0; k < kDwords; ++k)
+        u.w[k] = (uint32_t)__shfl_down((int)u.w[k], delta, 64);
+    return u.a;
+}
+
+// the reference's one-block routine (:99-141) over m < 128 values, by one thread
+template <typename A, typename Op> __device__ A ref_one_block(const A *v, int m)
+{
+    const int nw = (m + kRefWarp - 1) / kRefWarp;
+    A result{};
+    for (int w = 0; w < nw; ++w) {
+        A wres;
+        if ((w + 1) * kRefWarp < m) {
+            A t[kRefWarp];
+            for (int l = 0; l < kRefWarp; ++l)
+                t[l] = v[w * kRefWarp + l];
+            for (int width = kRefWarp / 2; width; width /= 2)
+                for (int l = 0; l < width; ++l)
+                    t[l] = Op::apply(t[l], t[l + width]);
+            wres = t[0];
+        } else {
+            wres = v[w * kRefWarp];
+            for (int i = 1; i < m - w * kRefWarp; ++i)
+                wres = Op::apply(wres, v[w * kRefWarp + i]);
+        }
+        result = w == 0 ? wres : Op::apply(result, wres);
+    }
+    return result;
+}
+
+template <typename T, typename Op, bool PACKED>
+__global__ __launch_bounds__(kOrdThreads) void reduce_ordered_kernel(const T *__restrict__ in, int64_t n,
+                                                                     int64_t stride, T init, T *__restrict__ out,
+                                                                     uint64_t *__restrict__ partials_raw,
+                                                                     unsigned *__restrict__ ticket)
+{
+    using A = typename AccOf<T, Op>::type;
+    using Word = typename WordsOf<A>::Word;
+    using Image = typename WordsOf<A>::Image;
+    constexpr int kWords = WordsOf<A>::kWords;
+    constexpr int E = (int)sizeof(T);
+    constexpr int V = 16 / E;                      // items per 16-byte packet
+    constexpr int LPR = kRefWarp / V;              // lanes that load one row piece of 32 items
+    constexpr int RPP = kOrdLoaders / LPR;         // rows per round of the loading lanes
+    constexpr int kBatch = RPP * kOrdRounds;       // rows parked in LDS at a time
+    // items per chain and buffer (the rows of a chain lie side by side).  Two more than a
+    // power of two: the scattered stores of a wavefront that parks its packets then fall
+    // on every LDS bank equally, and a pair of rows can still be read as one aligned piece
+    constexpr int kPitch = kBatch + 2;
+    // two buffers: the chains take one in while the next batch is parked in the other
+    __shared__ __attribute__((aligned(16))) T cols[2][kRefWarp][kPitch];
+    __shared__ A small[kRefBlock + 1 + kRefMaxGrid + 1];
+    __shared__ bool last_block;
+
+    const int tid = threadIdx.x;
+    const int64_t full = (n / kRefBlock) * kRefBlock;
+    int64_t ref_grid = full / kRefBlock;
+    if (ref_grid > kRefMaxGrid)
+        ref_grid = kRefMaxGrid;
+    const int64_t S = ref_grid * kRefBlock;        // chains; 0 when n < 128
+    const int warps = (int)(S / kRefWarp);         // = workgroups doing chains
+    const char *bytes = reinterpret_cast<const char *>(in);
+
+    if ((int)blockIdx.x < warps) {
+        // Workgroups are dealt to the eight XCDs in turn, and a workgroup reads the same 128
+        // bytes of every row: with warp w on workgroup w an XCD would see addresses that agree
+        // in bits 7 - 9, a fraction of its L2 channels.  Each XCD takes a run of neighbouring
+        // warps instead: a contiguous 4 KiB of every row.
+        int warp = (int)blockIdx.x;
+        if (warps % 8 == 0)
+            warp = (warp % 8) * (warps / 8) + warp / 8;
+        const int64_t c0 = (int64_t)warp * kRefWarp;                    // first chain of this warp
+        const int64_t nrows = (full - c0 + S - 1) / S;                   // items per chain
+        const bool loader = tid < kOrdLoaders;     // wavefronts 0..7; wavefront 8 runs the chains
+        const int lane = tid - kOrdLoaders;         // of the chain wavefront
+        const int my_row = tid / LPR, my_piece = tid % LPR;
+        A acc{};
+        union Pack {
+            nbh_u32x4 raw;
+            T item[V];
+        };
+        Pack held[2][kOrdRounds];                   // two batches on their way at any time
+        // Every round loads, without a branch around it (rows behind the last are replaced by
+        // the last: their copies are parked and never added): eight independent loads per lane
+        // that the hardware can have in flight together.
+        auto fetch = [&](Pack *into, int64_t first_row) {
+            if constexpr (PACKED) {
+#pragma unroll
+                for (int k = 0; k < kOrdRounds; ++k) {
+                    int64_t r = first_row + k * RPP + my_row;
+                    r = r < nrows ? r : nrows - 1;
+                    into[k].raw = nbh_load16<E, true>(in + (r * S + c0 + my_piece * V));
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < kOrdRounds; ++k) {
+                    int64_t r = first_row + k * RPP + my_row;
+                    r = r < nrows ? r : nrows - 1;
+                    const int64_t item = r * S + c0 + my_piece * V;
+#pragma unroll
+                    for (int j = 0; j < V; ++j)
+                        into[k].item[j] = *reinterpret_cast<const T *>(bytes + (item + j) * stride);
+                }
+            }
+        };
+        auto park = [&](const Pack *from, int buf) {  // lane (row, piece) holds V neighbouring chains' items of one row
+#pragma unroll
+            for (int k = 0; k < kOrdRounds; ++k)
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    cols[buf][my_piece * V + j][k * RPP + my_row] = from[k].item[j];
+        };
+        auto chains = [&](int buf, int64_t base) {
+            if (lane >= 0 && lane < kRefWarp) {
+                const T *__restrict__ mine = cols[buf][lane];
+                const int count = (int)((nrows - base < kBatch) ? nrows - base : kBatch);
+                int r = 0;
+                if (base == 0) {                    // a chain starts with its first value, not with an identity
+                    acc = (A)mine[0];
+                    r = 1;
+                }
+                if (r < count && (r & 1)) {
+                    acc = Op::apply(acc, (A)mine[r]);
+                    ++r;
+                }
+                struct alignas(2 * sizeof(T)) Two {
+                    T item[2];
+                };
+                const Two *__restrict__ pairs = reinterpret_cast<const Two *>(mine);
+                // two sets of registers take turns: while one is added up, the other is on its
+                // way from LDS (32 dwords a set, whatever the element size)
+                constexpr int U = (32 / E) < 1 ? 1 : (32 / E);   // pairs of rows per set
+                constexpr int G = 2 * U;                          // rows per set
+                auto read = [&](Two *into, int at) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u)
+                        into[u] = pairs[at / 2 + u];
+                };
+                auto add_up = [&](const Two *from) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        acc = Op::apply(acc, (A)from[u].item[0]);
+                        acc = Op::apply(acc, (A)from[u].item[1]);
+                    }
+                };
+                if (r + G <= count) {
+                    Two one[U], other[U];
+                    read(one, r);
+                    while (r + 3 * G <= count) {
+                        read(other, r + G);
+                        add_up(one);
+                        read(one, r + 2 * G);
+                        add_up(other);
+                        r += 2 * G;
+                    }
+                    if (r + 2 * G <= count) {
+                        read(other, r + G);
+                        add_up(one);
+                        add_up(other);
+                        r += 2 * G;
+                    } else {
+                        add_up(one);
+                        r += G;
+                    }
+                }
+                for (; r < count; ++r)
+                    acc = Op::apply(acc, (A)mine[r]);
+            }
+        };
+        // Two batches are on their way at any time, one per set of registers: a batch is parked
+        // as soon as it has arrived (the younger one still travelling), the batch after next is
+        // asked for into the registers just emptied, and the chains take the parked batch in
+        // meanwhile.  One barrier per batch: whoever parks into a buffer has passed the barrier
+        // the chains reached after reading it.  The steady-state loop always asks for both
+        // batches, so that the wait before each parking is for the older eight loads only
+        // (a load that is skipped on some path would make the compiler wait for all of them);
+        // the last one to three batches are taken outside it.
+        const int64_t nb = (nrows + kBatch - 1) / kBatch;
+        if (loader) {
+            fetch(held[0], 0);
+            fetch(held[1], kBatch);                 // rows behind the last repeat the last: harmless
+        }
+        int64_t b = 0;
+        for (; b + 3 < nb; b += 2) {
+            if (loader)
+                park(held[0], 0);
+            __syncthreads();
+            if (loader)
+                fetch(held[0], (b + 2) * kBatch);
+            else
+                chains(0, b * kBatch);
+            if (loader)
+                park(held[1], 1);
+            __syncthreads();
+            if (loader)
+                fetch(held[1], (b + 3) * kBatch);
+            else
+                chains(1, (b + 1) * kBatch);
+        }
+        if (loader)
+            park(held[0], 0);
+        __syncthreads();
+        if (loader) {
+            if (b + 2 < nb)
+                fetch(held[0], (b + 2) * kBatch);
+        } else {
+            chains(0, b * kBatch);
+        }
+        if (b + 1 < nb) {
+            if (loader)
+                park(held[1], 1);
+            __syncthreads();
+            if (!loader)
+                chains(1, (b + 1) * kBatch);
+        }
+        if (b + 2 < nb) {
+            if (loader)
+                park(held[0], 0);
+            __syncthreads();
+            if (!loader)
+                chains(0, (b + 2) * kBatch);
+        }
+        if (!loader) {                              // the chain wavefront, whole: the shuffles need its lanes
+#pragma unroll
+            for (int width = kRefWarp / 2; width; width /= 2) {
+                const A other = lane_below(acc, width);
+                if (lane < width)
+                    acc = Op::apply(acc, other);
+            }
+            if (lane == 0) {
+                Word *partials = reinterpret_cast<Word *>(partials_raw);
+                const Image img = WordsOf<A>::pack(acc);
+                Word before[kWords];
+#pragma unroll
+                for (int w = 0; w < kWords; ++w)
+                    before[w] = __hip_atomic_exchange(&partials[(int64_t)warp * kWords + w], img.w[w],
+                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int w = 0; w < kWords; ++w)
+                    asm volatile("" ::"v"(before[w]) : "memory");  // carried out before anyone goes on
+            }
+        }
+        __syncthreads();                            // the warp's result is published: the ticket may be drawn
+    }
+    if (gridDim.x > 1) {
+        if (tid == 0) {
+            const unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_block = (t == gridDim.x - 1);
+            if (last_block)
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        }
+        __syncthreads();
+        if (!last_block)
+            return;
+    }
+
+    // the small rest, laid out as small[0 .. 127]: the values behind `full`, small[128 ...]: the partials
+    const int m_tail = (int)(n - full);
+    A *tail = small, *part = small + kRefBlock + 1;
+    if (tid < m_tail)
+        tail[tid] = (A) * reinterpret_cast<const T *>(bytes + (full + tid) * stride);
+    if (tid < (int)ref_grid) {                      // block = (w0 op w2) op (w1 op w3)
+        const Word *partials = reinterpret_cast<const Word *>(partials_raw);
+        A w[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            Image img;
+#pragma unroll
+            for (int k = 0; k < kWords; ++k)
+                img.w[k] = __hip_atomic_load(&partials[((int64_t)tid * 4 + q) * kWords + k], __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+            w[q] = WordsOf<A>::unpack(img);
+        }
+        part[tid] = Op::apply(Op::apply(w[0], w[2]), Op::apply(w[1], w[3]));
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int np = (int)ref_grid;
+        if (ref_grid)
+            part[0] = Op::apply(part[0], (A)init);
+        if (m_tail) {
+            part[np] = ref_one_block<A, Op>(tail, m_tail);
+            if (!ref_grid)
+                part[0] = Op::apply(part[0], (A)init);
+            ++np;
+        }
+        const A result = np > 1 ? ref_one_block<A, Op>(part, np) : part[0];
+        out[0] = (T)result;
+        if (gridDim.x > 1)
+            __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+template <typename T, typename Op>
+int launch_ordered(const void *in, int64_t n, int64_t stride, const void *init, void *out, void *scratch,
+                   hipStream_t stream)
+{
+    const uintptr_t addr = (uintptr_t)in;
+    if (addr % sizeof(T) != 0 || ((uintptr_t)out) % sizeof(T) != 0 || stride % (int64_t)sizeof(T) != 0)
+        return (int)hipErrorInvalidValue;
+    int64_t ref_grid = n / kRefBlock;
+    if (ref_grid > kRefMaxGrid)
+        ref_grid = kRefMaxGrid;
+    const int64_t grid = ref_grid ? ref_grid * (kRefBlock / kRefWarp) : 1;  // one workgroup per reference warp
+    T init_value;
+    __builtin_memcpy(&init_value, init, sizeof(T));
+    unsigned *ticket = reinterpret_cast<unsigned *>(scratch);
+    uint64_t *partials = reinterpret_cast<uint64_t *>((char *)scratch + kHeaderBytes);
+    if (stride == (int64_t)sizeof(T) || n == 1)
+        hipLaunchKernelGGL((reduce_ordered_kernel<T, Op, true>), dim3((unsigned)grid), dim3(kOrdThreads), 0, stream,
+                           (const T *)in, n, (int64_t)sizeof(T), init_value, (T *)out, partials, ticket);
+    else
+        hipLaunchKernelGGL((reduce_ordered_kernel<T, Op, false>), dim3((unsigned)grid), dim3(kOrdThreads), 0, stream,
+                           (const T *)in, n, stride, init_value, (T *)out, partials, ticket);
+    return nbh_launch_status();
+}
+
+template <typename T> int launch_ordered_op(int op, const void *in, int64_t n, int64_t stride, const void *init,
+                                            void *out, void *scratch, hipStream_t s)
+{
+    switch (op) {
+    case NBH_ADD: return launch_ordered<T, OpAdd>(in, n, stride, init, out, scratch, s);
+    case NBH_MUL: return launch_ordered<T, OpMul>(in, n, stride, init, out, scratch, s);
+    default: break;
+    }
+    if constexpr (!IsCplx<T>::value) {
+        switch (op) {
+        case NBH_MAX: return launch_ordered<T, OpMax>(in, n, stride, init, out, scratch, s);
+        case NBH_MIN: return launch_ordered<T, OpMin>(in, n, stride, init, out, scratch, s);
+        default: break;
+        }
+    }
+    return (int)hipErrorInvalidValue;
+}
+
 template <typename T, typename Op>
 int launch(const void *in, int64_t n, int64_t stride, const void *init, void *out, void *scratch,
            hipStream_t stream)
@@ -505,6 +877,26 @@ int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, 
     case NBH_C64: return launch_op_complex<Cplx<float>>(op, in, n, in_stride, init, out, scratch, s);
     case NBH_C128: return launch_op_complex<Cplx<double>>(op, in, n, in_stride, init, out, scratch, s);
     default: return (int)hipErrorInvalidValue;
+    }
+}
+
+int nbh_reduce_ordered(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
+                       void *scratch, size_t scratch_bytes, nbh_stream_t stream)
+{
+    if (!in || !init || !out || !scratch || n < 1 || scratch_bytes < kScratchBytes ||
+        ((uintptr_t)scratch) % 8 != 0)
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = nbh_hip_stream(stream);
+    nbh_stream_report report(s);
+    switch (dtype) {
+    case NBH_F32: return launch_ordered_op<float>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_F64: return launch_ordered_op<double>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_F16: return launch_ordered_op<Half>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_C64: return launch_ordered_op<Cplx<float>>(op, in, n, in_stride, init, out, scratch, s);
+    case NBH_C128: return launch_ordered_op<Cplx<double>>(op, in, n, in_stride, init, out, scratch, s);
+    default:
+        // integers and booleans: every order of association gives the same bits
+        return nbh_reduce(op, dtype, in, n, in_stride, init, out, scratch, scratch_bytes, stream);
     }
 }
 
