@@ -10,8 +10,9 @@ are resident in HBM before the clock starts.  Prints ONE JSON line.
 
 Without --workload the same line carries an `others` array with every other
 benchmark configuration measured in the same process: reduce_f32_max,
-reduce_f64_sum, reduce_i64_sum, transpose_f32, transpose_f64, transpose_i16,
-rng_init, rng_uniform_f32, rng_normal_f64, batched_reduce.  --workload NAME measures
+reduce_f64_sum, reduce_i64_sum, reduce_f32_functor (a translated functor),
+reduce_f32_sum_reference_order (the reference's association order), transpose_f32,
+transpose_f64, transpose_i16, rng_init, rng_uniform_f32, rng_normal_f64, batched_reduce.  --workload NAME measures
 just one of them (or copy_f32, the counter calibration kernel) as the headline.
 """
 
@@ -48,6 +49,10 @@ MEASURED_TRAFFIC = {
     "reduce_f64_sum": 1073820062,
     "reduce_i64_sum": 2147534810,
     "transpose_i16": 1073901040,      # profiles/transpose_packets_f32_16384sq.txt, last section
+    # profiles/reduce_ordered_kernel_f32_sum_2p28.txt: 1 073 919 663 B fetched + 16 441 B written
+    "reduce_f32_sum_reference_order": 1073936104,
+    # profiles/reduce_kernel_other_dtypes_and_batched.txt: 1 073 905 148 B fetched + 32 821 B written
+    "reduce_f32_functor": 1073937969,
     "rng_normal_f64": 2684437180,
     "rng_init": 269594109,
 }
@@ -150,6 +155,10 @@ def _workload(name, cuda):
             # a functor without a kernel of its own: translated and compiled at run time
             host = rng.standard_normal(2**28, dtype=np.float32)
             desc = "cuda.reduce fp32 with lambda a, b: sqrt(a*a + b*b) (translated functor), 2^28 elements N(0,1), seed 1"
+        elif name == "reduce_f32_sum_reference_order":
+            # the same sum with the association order of the reference's kernels: its bits
+            host = rng.standard_normal(2**28, dtype=np.float32)
+            desc = "cuda.reduce fp32 sum in the reference's association order (bit-identical result), 2^28 elements N(0,1), seed 1"
         elif name == "reduce_f32_sum" or name == "reduce_f32_max":
             host = rng.standard_normal(2**28, dtype=np.float32)
             desc = "cuda.reduce fp32 %s, 2^28 elements N(0,1), seed 1" % ("sum" if name.endswith("sum") else "max")
@@ -171,6 +180,9 @@ def _workload(name, cuda):
         if name.endswith("functor"):
             red = cuda.Reduce(_hypot)
             kernel = "nbh_custom_reduce"
+        if name.endswith("reference_order"):
+            red = cuda.Reduce(lambda a, b: a + b, reference_order=True)
+            kernel = "reduce_ordered_kernel"
 
         def step(i):
             red(bufs[i & 1], res=res, init=init, stream=stream)
@@ -301,11 +313,14 @@ TRAFFIC_SOURCE = {
     "reduce_f64_sum": "profiles/hbm_counters_other_workloads.txt",
     "reduce_i64_sum": "profiles/hbm_counters_other_workloads.txt",
     "transpose_i16": "profiles/transpose_packets_f32_16384sq.txt",
+    "reduce_f32_sum_reference_order": "profiles/reduce_ordered_kernel_f32_sum_2p28.txt",
+    "reduce_f32_functor": "profiles/reduce_kernel_other_dtypes_and_batched.txt",
     "rng_normal_f64": "profiles/hbm_counters_other_workloads.txt",
     "rng_init": "profiles/hbm_counters_other_workloads.txt",
 }
 
-OTHER_WORKLOADS = ["reduce_f32_max", "reduce_f64_sum", "reduce_i64_sum", "reduce_f32_functor", "transpose_f32", "transpose_f64",
+OTHER_WORKLOADS = ["reduce_f32_max", "reduce_f64_sum", "reduce_i64_sum", "reduce_f32_functor", "reduce_f32_sum_reference_order",
+                   "transpose_f32", "transpose_f64",
                    "transpose_i16", "rng_init", "rng_uniform_f32", "rng_normal_f64", "batched_reduce"]
 
 
