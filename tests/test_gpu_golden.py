@@ -58,6 +58,12 @@ def test_reductions_against_reference_order_values(case):
     assert abs(float(got) / float(want) - 1) <= 4 * n * eps                               # tolerance: 4 n eps, relative
     for op, value in case["int64_uniform_pm_2_20"].items():
         assert int(cuda.Reduce(ops[op])(i, init=3)) == value
+    # in the reference's association order the device reproduces the recorded bits
+    for op, bits in case["float32_standard_normal"].items():
+        got = cuda.Reduce(ops[op], reference_order=True)(f, init=0.5)
+        assert int(np.asarray(got).view(np.uint32)) == bits, (n, op)
+    got = cuda.Reduce(lambda a, b: a * b, reference_order=True)(near_one, init=1)
+    assert int(np.asarray(got).view(np.uint32)) == case["float32_near_one_product"], n
 
 
 def test_closed_forms_on_the_device():
