@@ -431,7 +431,7 @@ def main():
         others = []
         for other in OTHER_WORKLOADS:
             _release_device_memory(cuda)
-            steps, warmup = (3, 1) if other == "batched_reduce" else (min(args.steps, 50), min(args.warmup, 5))
+            steps, warmup = (10, 2) if other == "batched_reduce" else (min(args.steps, 50), min(args.warmup, 5))
             print("bench: %s ..." % other, file=sys.stderr, flush=True)
             others.append(measure(cuda, other, steps, warmup, 0 if args.no_cpu_baseline else 2.0))
         line["others"] = others
