@@ -939,9 +939,10 @@ class IpcHandle:
         self.base, self.handle, self.size = base, handle, size
         self.source_info, self.offset = source_info, offset
         self._mapping = None        # MemoryPointer over the imported allocation while open
+        self._staged = False        # open_staged() happened and close() has not yet
 
     def _refuse_if_open(self):
-        if self._mapping is not None:
+        if self._mapping is not None or self._staged:
             raise ValueError("IpcHandle is already opened")
 
     def _need_source_info(self):
@@ -954,11 +955,30 @@ class IpcHandle:
         return self.source_info == here or context.can_access_peer(Device.from_identity(self.source_info).id)
 
     def open_staged(self, context):
-        """Copy through the exporting device when the importer cannot reach it.  That
-        needs a second device in the importing process, which this build never has."""
+        """For an importing device that cannot reach the exporting one: map the memory on
+        the exporting device, copy it into a fresh allocation of `context` and unmap it
+        again (reference :1445-1482).  The result is a COPY, owned by the caller; close()
+        then has nothing left to undo.  The copy between two devices is the runtime's
+        (direct if they are peers, through the host if not)."""
+        from numba_cuda_amd.cudadrv import devices
         self._need_source_info()
         self._refuse_if_open()
-        raise NotImplementedError("staged IPC between two devices is not part of this build")
+        if self.base is not None:
+            raise ValueError("opening IpcHandle from original process")
+        wanted = self.offset + self.size
+        if wanted >= IPC_ALLOCATION_LIMIT:
+            raise ValueError("allocations of 2 GiB or more cannot be shared between processes")
+        source = Device.from_identity(self.source_info)
+        with devices.gpus[source.id]:
+            mapping = devices.get_context().open_ipc_handle(self.handle, wanted)
+        try:
+            copy = context.memalloc(self.size)
+            device_to_device(copy, mapping.view(self.offset), self.size)
+        finally:
+            with devices.gpus[source.id]:
+                driver.nbh_ipc_close(mapping.handle)
+        self._staged = True
+        return copy
 
     def open_direct(self, context):
         self._refuse_if_open()
@@ -984,6 +1004,9 @@ class IpcHandle:
                                          dtype=dtype, gpu_data=memory)
 
     def close(self):
+        if self._staged and self._mapping is None:     # a staged open left a copy, not a mapping
+            self._staged = False
+            return
         if self._mapping is None:
             raise ValueError("IpcHandle not opened")
         mapping, self._mapping = self._mapping, None

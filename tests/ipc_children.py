@@ -53,3 +53,19 @@ def reduce_transpose_and_write(ipcarr, parent_pid):
         darr[0, :] = -1.0
         cuda.synchronize()
     return float(total), flipped
+
+
+def read_staged(handle, device_num, parent_pid):
+    """The reference's staged case (tests/cudapy/test_ipc.py:177-191): a copy of the shared
+    memory made through the exporting device; writes to the copy stay in this process."""
+    assert os.getpid() != parent_pid
+    with cuda.gpus[device_num]:
+        ctx = cuda.devices.get_context()
+        copy = handle.open_staged(ctx)
+        count = handle.size // np.dtype(np.intp).itemsize
+        host = np.zeros(count, dtype=np.intp)
+        cuda.driver.device_to_host(host, copy, size=handle.size)
+        cuda.driver.device_memset(copy, 0xFF, handle.size)      # must not reach the exporter
+        cuda.synchronize()
+        handle.close()
+    return host

@@ -84,6 +84,18 @@ def test_array_handle(worker, index, foreign):
     np.testing.assert_array_equal(fut.result(timeout=TIMEOUT), expect)
 
 
+def test_staged_open_on_every_device(worker):
+    """tests/cudapy/test_ipc.py:212-233: the importer copies through the exporting device."""
+    _say("staged")
+    arr = np.arange(10, dtype=np.intp)
+    devarr = cuda.to_device(arr)
+    ipch = cuda.current_context().get_ipc_handle(devarr.gpu_data)
+    for device_num in range(len(cuda.gpus)):
+        fut = worker.submit(ipc_children.read_staged, ipch, device_num, parent_pid=os.getpid())
+        np.testing.assert_array_equal(fut.result(timeout=TIMEOUT), arr)
+    np.testing.assert_array_equal(devarr.copy_to_host(), arr)       # the child only wrote to its copy
+
+
 def test_the_other_process_computes_on_and_writes_to_the_shared_array(worker):
     _say("compute in the other process")
     rng = np.random.default_rng(5)

@@ -127,8 +127,20 @@ def test_other_cases(fake_gpu, monkeypatch):
     elsewhere.source_info = {"pci_domain_id": 9, "pci_bus_id": 9, "pci_device_id": 9}
     with pytest.raises(RuntimeError, match="No device of .* is found"):
         elsewhere.open(ctx)
-    with pytest.raises(NotImplementedError, match="staged IPC"):
-        pickle.loads(pickle.dumps(ipch)).open_staged(ctx)
+    # staged: a copy through the exporting device (here the same one), owned by the caller
+    with pytest.raises(ValueError, match="opening IpcHandle from original process"):
+        ipch.open_staged(ctx)
+    imported = pickle.loads(pickle.dumps(ipch))
+    copy = imported.open_staged(ctx)
+    got = np.zeros(4)
+    drv.device_to_host(got, copy, got.nbytes)
+    np.testing.assert_array_equal(got, np.arange(4.0))
+    assert copy.device_pointer_value != devarr.gpu_data.device_pointer_value
+    with pytest.raises(ValueError, match="IpcHandle is already opened"):
+        imported.open_staged(ctx)
+    imported.close()                                  # nothing to unmap; the copy lives on
+    with pytest.raises(ValueError, match="IpcHandle not opened"):
+        imported.close()
     monkeypatch.setattr(drv.sys, "platform", "win32")
     with pytest.raises(OSError, match="OS does not support CUDA IPC"):
         ctx.get_ipc_handle(devarr.gpu_data)
