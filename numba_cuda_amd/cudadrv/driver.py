@@ -33,7 +33,14 @@ from numba_cuda_amd import _lib
 from numba_cuda_amd import _build
 
 if _build.hostbuf_needs_building():      # not built yet, or older than its source: one gcc call, about a second
-    _build.build_hostbuf()
+    try:
+        _build.build_hostbuf()
+    except Exception:
+        import os as _os
+        if not _os.path.exists(_build.HOSTBUF_PATH):
+            raise
+        # an older build is there and cannot be replaced (no compiler, read-only tree):
+        # it lacks what was added since, and the callers of those parts check for them
 from numba_cuda_amd import _hostbuf
 from numba_cuda_amd.core import config
 from numba_cuda_amd.core.errors import CudaDriverError, CudaSupportError  # noqa: F401

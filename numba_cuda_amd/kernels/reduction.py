@@ -408,7 +408,7 @@ _Stream = _driver.Stream
 _PER_THREAD = _driver.HIP_STREAM_PER_THREAD
 _thread_state = devices._runtime._tls
 _call_reduce = _driver._hostbuf.call_reduce
-_reduce_into = _driver._hostbuf.reduce_into
+_reduce_into = getattr(_driver._hostbuf, "reduce_into", lambda *args: NotImplemented)   # absent from an older build
 
 def _entry_address(lib):
     """Address of the library's nbh_reduce for call_reduce, kept on the library object
