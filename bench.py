@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E published peak
 # (see profiles/); filled in per workload once measured, else None
 MEASURED_TRAFFIC = {
     # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 777 931 B fetched + 32 823 B written
-    "reduce_f32_sum": 1073810755,
+    "reduce_f32_sum": 1073817508,
     # profiles/copy_flat_f32_2p28.txt: the calibration kernel itself
     "copy_f32": 2147483648,
     # profiles/transpose_packets_f32_16384sq.txt: 1 073 761 075 B fetched + 1 074 512 910 B written
@@ -45,9 +45,9 @@ MEASURED_TRAFFIC = {
     # profiles/transpose_sheared_f64_12345x6789.txt: 768 287 439 B fetched + 670 489 125 B written
     "transpose_f64": 1438776564,
     # profiles/hbm_counters_other_workloads.txt
-    "reduce_f32_max": 1073822046,
-    "reduce_f64_sum": 1073820062,
-    "reduce_i64_sum": 2147534810,
+    "reduce_f32_max": 1073827256,
+    "reduce_f64_sum": 1073823652,
+    "reduce_i64_sum": 2147537460,
     "transpose_i16": 1073901040,      # profiles/transpose_packets_f32_16384sq.txt, last section
     # profiles/reduce_ordered_kernel_f32_sum_2p28.txt: 1 073 919 663 B fetched + 16 441 B written
     "reduce_f32_sum_reference_order": 1073936104,

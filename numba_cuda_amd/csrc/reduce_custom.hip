@@ -19,7 +19,8 @@
 // associative and commutative.
 //
 // One launch of `nbh_custom_reduce`, shaped like nbh_reduce's kernel: 512-thread workgroups,
-// two per compute unit, each streaming one contiguous slice; one partial per workgroup in
+// two per compute unit, each streaming one contiguous slice (large inputs: 16 KiB pieces
+// dealt out round robin); one partial per workgroup in
 // the scratch buffer; the workgroup that draws the last ticket folds the partials, applies
 // `init` and writes `out`.  Ticket and partial slots are those of nbh_reduce's scratch
 // buffer, used the same way (the ticket is handed back at zero), so one buffer serves both
@@ -38,6 +39,7 @@ namespace {
 
 constexpr int kBlock = 512;               // threads per workgroup; the device source says the same
 constexpr int kUnroll = 4;
+constexpr int64_t kPiecePackets = 2 * kBlock;  // a dealt piece; the device source says the same
 constexpr int kGridPerCU = 2;
 constexpr int kMaxGrid = 4096;            // partial slots in nbh_reduce's scratch buffer
 constexpr size_t kHeaderBytes = 256;      // the ticket lives here
@@ -156,6 +158,7 @@ __device__ __forceinline__ T nbh_op(T a, T b)
 
 constexpr int kItems = 16 / (int)sizeof(T);     // elements per 16-byte packet
 constexpr int kThreads = 512, kWaves = 8, kUnroll = 4;
+constexpr long long kPiece = 2 * kThreads;      // packets per dealt piece
 union nbh_packet { nbh_u32x4 raw; T item[kItems]; };
 union nbh_slot { nbh_u64 word; T value; };
 
@@ -224,6 +227,7 @@ __device__ __forceinline__ void nbh_fold_workgroup(T &acc, bool &have)
 // atomics are carried out where all of them look).
 // packed != 0: items [head, head + units * kItems) are `units` aligned packets; the `head`
 // items in front and the fewer than kItems behind are taken by single lanes of workgroup 0.
+// packed == 2: large inputs, read piece by piece instead of slice by slice (see there).
 // packed == 0: `units` items, `stride` bytes apart.
 extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce(const char *__restrict__ in, long long n,
                                                                    long long head, long long units,
@@ -242,7 +246,43 @@ extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce(const char *
     T acc = T();
     bool have = false;
     long long i = begin + tid;
-    if (packed) {
+    if (packed == 2) {
+        // pieces of 2 * kThreads packets dealt out round robin (piece q of a round to the
+        // workgroup whose XCD comes q / (grid / 8)-th): the workgroups read one moving
+        // window; the caller sees to it that each of them gets two pieces or more
+        const nbh_u32x4 *__restrict__ p = reinterpret_cast<const nbh_u32x4 *>(in + head * (long long)sizeof(T));
+        const long long grid = gridDim.x, pieces = units / kPiece;
+        const long long first = grid % 8 == 0 ? (long long)(blockIdx.x % 8) * (grid / 8) + blockIdx.x / 8
+                                              : (long long)blockIdx.x;
+        const nbh_u32x4 *__restrict__ q = p + first * kPiece + tid;
+        nbh_u32x4 c0 = __builtin_nontemporal_load(q), c1 = __builtin_nontemporal_load(q + kThreads);
+        q += grid * kPiece;
+        nbh_u32x4 n0 = __builtin_nontemporal_load(q), n1 = __builtin_nontemporal_load(q + kThreads);
+        acc = nbh_op(nbh_fold_packet(c0), nbh_fold_packet(c1));
+        have = true;
+        c0 = n0;
+        c1 = n1;
+        for (long long c = first + 2 * grid; c < pieces; c += grid) {
+            q += grid * kPiece;
+            n0 = __builtin_nontemporal_load(q);
+            n1 = __builtin_nontemporal_load(q + kThreads);
+            acc = nbh_op(acc, nbh_op(nbh_fold_packet(c0), nbh_fold_packet(c1)));
+            c0 = n0;
+            c1 = n1;
+        }
+        acc = nbh_op(acc, nbh_op(nbh_fold_packet(c0), nbh_fold_packet(c1)));
+        if (blockIdx.x == gridDim.x - 1)  // less than a piece of whole packets is left over
+            for (long long k = pieces * kPiece + tid; k < units; k += kThreads)
+                acc = nbh_op(acc, nbh_fold_packet(__builtin_nontemporal_load(p + k)));
+        if (blockIdx.x == 0) {
+            const T *__restrict__ items = reinterpret_cast<const T *>(in);
+            const long long tail_begin = head + units * kItems;
+            if (tid < head)
+                nbh_take(acc, have, items[tid]);
+            else if (tail_begin + (tid - head) < n)
+                nbh_take(acc, have, items[tail_begin + (tid - head)]);
+        }
+    } else if (packed) {
         const nbh_u32x4 *__restrict__ p = reinterpret_cast<const nbh_u32x4 *>(in + head * (long long)sizeof(T));
         if (i < end) {
             acc = nbh_fold_packet(__builtin_nontemporal_load(p + i));
@@ -484,7 +524,8 @@ extern "C" int nbh_reduce_custom(void *handle, const void *in, int64_t n, int64_
 
     const char *in_arg = static_cast<const char *>(in);
     long long n_arg = n, stride_arg = in_stride;
-    int packed_arg = packed;
+    // from sixteen pieces per workgroup on, the pieces are dealt out (as in nbh_reduce)
+    int packed_arg = (packed && units / kPiecePackets >= 16 * grid) ? 2 : packed;
     uint64_t *partials = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kHeaderBytes);
     unsigned *ticket = reinterpret_cast<unsigned *>(scratch);
     // `init` travels as a kernel argument: the launch copies the element it points to
