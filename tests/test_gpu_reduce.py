@@ -385,6 +385,50 @@ def test_fullsize_int64_sum_2_pow_28_bit_exact():
     assert got == cref.tree("add", a) == a.sum()
 
 
+@pytest.mark.parametrize("dtype,items,skip", [
+    (np.int8, 150_000_011, 3), (np.uint16, 80_000_003, 1), (np.int32, 40_000_001, 3),
+    (np.int64, 20_000_003, 1), (np.float64, 25_000_007, 1), (np.complex128, 10_000_019, 0),
+    (np.float32, 35_000_017, 2), (np.int32, 33_554_432 + 1024 * 4 * 5, 0)])
+def test_large_inputs_of_awkward_length_and_start(dtype, items, skip):
+    """From 128 MiB on the input is read in 16 KiB pieces dealt out to the workgroups: lengths
+    that leave part of a piece and part of a 16-byte packet over, views that start off a
+    16-byte boundary, every item size.  Integers wrap, so every association gives the same
+    bits; the floating-point data are small integers whose sums are exact in any order."""
+    rng = np.random.default_rng(items)
+    dt = np.dtype(dtype)
+    _say("large", dt.name, items, skip)
+    if dt.kind in "iu":
+        info = np.iinfo(dt)
+        host = rng.integers(info.min, info.max, items, dtype=dt, endpoint=True)
+    elif dt.kind == "c":
+        host = (rng.integers(-8, 8, items) + 1j * rng.integers(-8, 8, items)).astype(dt)
+    else:
+        host = rng.integers(-8, 8, items).astype(dt)
+    whole = cuda.to_device(host)
+    dev, ref = whole[skip:], host[skip:]
+    assert dev.nbytes >= 128 << 20
+    got = sum_reduce(dev)
+    if dt.kind in "iu":
+        assert got == ref.sum(dtype=dt)
+    elif dt == np.float32:   # partial sums stay far below 2^24 in practice but nothing bounds them
+        assert abs(float(got) - float(ref.sum(dtype=np.float64))) <= 2 * ref.size * np.finfo(dt).eps * float(np.abs(ref).sum(dtype=np.float64))
+    else:
+        assert got == ref.sum()
+    if dt.kind != "c":
+        # a maximum in the last item and a minimum in the first: the edges of the range count
+        host[-1], host[skip] = host.max(), host.min()
+        whole[items - 1:items] = host[-1:]
+        whole[skip:skip + 1] = host[skip:skip + 1]
+        lo, hi = (np.iinfo(dt).min, np.iinfo(dt).max) if dt.kind in "iu" else (-np.inf, np.inf)
+        assert cuda.Reduce(lambda x, y: max(x, y))(dev, init=lo) == ref.max()
+        assert cuda.Reduce(lambda x, y: min(x, y))(dev, init=hi) == ref.min()
+        marked = host.copy()
+        spot = items - 1 - (items - skip) % 4096 // 2   # inside what is left over behind the last piece
+        marked[spot] = hi if dt.kind in "iu" else 1000
+        whole[spot:spot + 1] = marked[spot:spot + 1]
+        assert cuda.Reduce(lambda x, y: max(x, y))(dev, init=lo) == marked[skip:].max()
+
+
 @pytest.mark.parametrize("n_min,n_max,calls", [(5000, 3_000_000, 3000), (2_200_000, 9_000_000, 1500)])
 def test_back_to_back_reductions_never_see_stale_partials(n_min, n_max, calls):
     """Thousands of launches reuse one scratch buffer per stream with different

@@ -102,6 +102,25 @@ def test_closed_forms_at_2p24():
     assert got == bool(flags.sum() & 1) and isinstance(got, np.bool_)
 
 
+@pytest.mark.parametrize("dtype,items,skip", [(np.int32, 40_000_001, 3), (np.uint16, 80_000_003, 1),
+                                              (np.int64, 20_000_003, 1), (np.uint8, 150_000_011, 5)])
+def test_closed_forms_on_large_inputs_of_awkward_length_and_start(dtype, items, skip):
+    """From 128 MiB on the translated kernel reads 16 KiB pieces dealt out to the workgroups:
+    lengths that leave part of a piece and of a packet over, starts off a 16-byte boundary."""
+    rng = np.random.default_rng(items)
+    info = np.iinfo(dtype)
+    data = rng.integers(info.min, info.max, items, dtype=dtype, endpoint=True)
+    d = cuda.to_device(data)[skip:]
+    ref = data[skip:]
+    assert d.nbytes >= 128 << 20
+    _say("large sum_plus_one", np.dtype(dtype), items, skip)
+    got = cuda.Reduce(FC.BY_NAME["sum_plus_one"].functor)(d, init=7)
+    total = int(np.sum(ref.astype(np.uint64), dtype=np.uint64))       # modulo 2^64
+    assert got == _wrap(total + 7 + ref.size, dtype)
+    got = cuda.Reduce(FC.BY_NAME["xor_and_flip"].functor)(d, init=5)
+    assert got == _wrap(int(np.bitwise_xor.reduce(ref)) ^ 5 ^ (ref.size & 1), dtype)
+
+
 def test_float16_and_booleans():
     rng = np.random.default_rng(16)
     x = (rng.standard_normal(5000) * 100).astype(np.float16)
