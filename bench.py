@@ -34,8 +34,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E published peak
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (see profiles/); filled in per workload once measured, else None
 MEASURED_TRAFFIC = {
-    # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 777 931 B fetched + 32 823 B written
-    "reduce_f32_sum": 1073817508,
+    # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 783 602 B fetched + 32 821 B written
+    "reduce_f32_sum": 1073816423,
     # profiles/copy_flat_f32_2p28.txt: the calibration kernel itself
     "copy_f32": 2147483648,
     # profiles/transpose_packets_f32_16384sq.txt: 1 073 761 075 B fetched + 1 074 512 910 B written

@@ -269,6 +269,7 @@ extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce(const char *
             acc = nbh_op(acc, nbh_op(nbh_fold_packet(c0), nbh_fold_packet(c1)));
             c0 = n0;
             c1 = n1;
+            __syncthreads();  // the wavefronts ask for a piece together, as one run of 16 KiB
         }
         acc = nbh_op(acc, nbh_op(nbh_fold_packet(c0), nbh_fold_packet(c1)));
         if (blockIdx.x == gridDim.x - 1)  // less than a piece of whole packets is left over
