@@ -13,7 +13,7 @@
 //     per lane in flight).  2^28 float32: 153.6 us with one contiguous slice per
 //     workgroup, 148 - 149 us dealt with a workgroup barrier per piece (the memory serves one moving front better than 512
 //     separate streams; many short-lived workgroups that read a piece each come to 143 us
-//     but need a partial and a ticket each, and tickets cost 12 ns apiece).
+//     but need a partial and a ticket each: 12 ns per workgroup with all tickets on one address).
 //   * inputs too small for two pieces per workgroup are cut into one contiguous slice
 //     per workgroup instead, kUnroll independent 16-byte loads in flight per lane
 //   * lanes fold into per-lane accumulators, a wavefront folds with four DPP
