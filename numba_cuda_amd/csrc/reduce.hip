@@ -4,18 +4,20 @@
 //   * the input is read once with 128-bit loads; the few elements in front of the
 //     first 16-byte boundary and behind the last whole vector are picked up by
 //     single lanes of workgroup 0
-//   * large inputs are cut into pieces of 16 KiB that are dealt out to the workgroups
-//     (8 wavefronts, two workgroups per compute unit) round robin, so that at any moment
-//     all of them read one window of a few MiB that moves through the input: piece p of
-//     a round goes to the workgroup whose XCD comes p / (grid / 8)-th, which gives every
-//     XCD one run of consecutive pieces per round; a workgroup has the loads of its next
-//     piece in flight while it adds the current one (non-temporal 16-byte loads, four
-//     per lane in flight).  2^28 float32: 153.6 us with one contiguous slice per
-//     workgroup, 148 - 149 us dealt with a workgroup barrier per piece (the memory serves one moving front better than 512
-//     separate streams; many short-lived workgroups that read a piece each come to 143 us
-//     but need a partial and a ticket each: 12 ns per workgroup with all tickets on one address).
-//   * inputs too small for two pieces per workgroup are cut into one contiguous slice
-//     per workgroup instead, kUnroll independent 16-byte loads in flight per lane
+//   * inputs from 128 MiB on are cut into pieces of 16 KiB that are dealt out to the
+//     workgroups (8 wavefronts, two workgroups per compute unit) round robin, so that at
+//     any moment all of them read one window of a few MiB that moves through the input:
+//     piece p of a round goes to the workgroup whose XCD comes p / (grid / 8)-th, which
+//     gives every XCD one run of consecutive pieces per round; a workgroup has the loads
+//     of its next piece in flight while it adds the current one (non-temporal 16-byte
+//     loads, four per lane in flight) and meets at a barrier after every piece, so that a
+//     piece is asked for as one run.  2^28 float32: 153.6 us with one contiguous slice per
+//     workgroup, 149.1 us dealt - the memory serves one moving front better than 512
+//     separate streams.  (Many short-lived workgroups that read a piece each come to
+//     143 us, but each needs a partial and a ticket: 12 ns per workgroup with all tickets
+//     on one address, and no cheaper with the tickets spread out.)
+//   * smaller inputs are cut into one contiguous slice per workgroup instead, kUnroll
+//     independent 16-byte loads in flight per lane
 //   * lanes fold into per-lane accumulators, a wavefront folds with four DPP
 //     steps inside each row of 16 lanes plus three scalar combines of the four row
 //     totals, the workgroup folds its wavefront totals through LDS
