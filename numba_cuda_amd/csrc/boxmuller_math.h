@@ -1,9 +1,14 @@
 // The two transcendental steps of Box-Muller, specialised to the arguments the
-// generators produce, each within one unit in the last place of double:
+// generators produce:
 //
 //   bm_log_f32(u)  natural logarithm of a float32 in (0, 1] (any positive normal
-//                  float32 works), evaluated in double; u == 0 gives -infinity.
-//   bm_cos_2pi(x)  cosine of a double in [0, 6.2832], i.e. of 2*pi*u.
+//                  float32 works), evaluated in double to within 0.52 units in the last
+//                  place (4.5 for u between 1/2 and 1, where terms cancel) - its callers
+//                  round it to float32, and for EVERY float32 in [2^-53, 1] (all a
+//                  generator can produce besides 0) that float32 is the one the correctly
+//                  rounded double logarithm rounds to; u == 0 gives -infinity.
+//   bm_cos_2pi(x)  cosine of a double in [0, 6.2832], i.e. of 2*pi*u, within one unit
+//                  in the last place of double.
 //   bm_sqrt_pos(a) square root for the range that occurs.
 //
 // The general-purpose library routines spend most of their time on cases that
@@ -32,6 +37,12 @@ namespace bm {
 // and the table holds q_j = RN(1 / c_j) and t_j = -log(q_j) as a double-double, so that
 //     log(m) = t_j + log1p(r),  r = m * q_j - 1  (|r| <= 2^-8)
 // holds exactly.  t_hi keeps 42 fractional bits: e * ln2_hi + t_hi is then exact.
+// Nothing is carried in two parts beyond that: a compensated evaluation (r as a sum of
+// two doubles, error-free addition of the leading terms) is good to 0.513 units in the
+// last place at 20 double-precision operations; the 12 below lose up to 4.5 where u is
+// just below 1, and a sweep over all 444 596 224 possible arguments
+// (tests/boxmuller_math_check.cpp) shows that no float32 rounding moves.  (One table word per run instead of two, or ln 2 in one
+// piece, moves one of them.)
 // (The table also carries the two coefficient sets of the cosine, see below: it is the
 // one block of constants the generators keep in LDS.)
 struct LogTable {
@@ -93,28 +104,19 @@ BM_FN double log_positive_f32(float u, const LogTable *__restrict__ tab)
     std::memcpy(&mf, &mbits, 4);
 #endif
     const double m = (double)mf, fe = (double)e;
-    // r + r_lo = m * q_j - 1 exactly: where t_j is small, r is as large as the result
-    // and its own rounding would show
-    const double q = tab->q[j];
-    const double mq = m * q;
-    const double r_lo = __builtin_fma(m, q, -mq);
-    const double r = mq - 1.0;
-    // log1p(r) - r, |r| <= 2^-8: the r^8 / 8 term is below 2^-67
-    double p = __builtin_fma(r, 1.0 / 7.0, -1.0 / 6.0);
-    p = __builtin_fma(r, p, 1.0 / 5.0);
+    // r = RN(m * q_j - 1): one rounding, relative to r itself
+    const double r = __builtin_fma(m, tab->q[j], -1.0);
+    // log1p(r) - r, |r| <= 2^-8: the r^7 / 7 term is below 2^-58
+    double p = __builtin_fma(r, -1.0 / 6.0, 1.0 / 5.0);
     p = __builtin_fma(r, p, -1.0 / 4.0);
     p = __builtin_fma(r, p, 1.0 / 3.0);
     p = __builtin_fma(r, p, -0.5);
     p = (r * r) * p;
-    p = __builtin_fma(-r, r_lo, p);                    // d/dr (log1p(r) - r) = -r to first order
     const double ln2_hi = 0x1.62e42feep-1;             // 32 bits of ln 2
     const double ln2_lo = 0x1.a39ef35793c76p-33;       // ln 2 - ln2_hi
     const double hi = __builtin_fma(fe, ln2_hi, tab->t_hi[j]);  // exact
-    // s + err = hi + r exactly: hi is zero (run of 1.0, e = 0) or |hi| > |r|
-    const double s = hi + r;
-    const double err = r - (s - hi);
-    const double lo = ((__builtin_fma(fe, ln2_lo, tab->t_lo[j]) + r_lo) + p) + err;
-    return s + lo;
+    const double lo = __builtin_fma(fe, ln2_lo, tab->t_lo[j]) + p;
+    return hi + (r + lo);                              // the small terms first
 }
 
 BM_FN double bm_log_f32(float u, const LogTable *__restrict__ tab)

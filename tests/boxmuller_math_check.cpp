@@ -3,8 +3,12 @@
 // result and the number of inputs whose rounding to float32 differs from the
 // rounding of the long-double value.  Built and run by tests/test_boxmuller_math.py.
 #include "boxmuller_math.h"
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
+#include <thread>
+#include <vector>
 
 static double ulp_of(long double want)
 {
@@ -40,6 +44,38 @@ int main(int argc, char **argv)
     {
         const double one = bm::bm_log_f32(1.0f, &tab), zero = bm::bm_log_f32(0.0f, &tab);
         printf("log edge: log(1)=%g signbit=%d log(0)=%g\n", one, (int)std::signbit(one), zero);
+    }
+
+    // logarithm, what its callers use: the float32 it rounds to, for every float32 a generator
+    // can produce besides zero - exponents -53 ... -1, every mantissa (second argument "all";
+    // eight threads, two seconds).  The yardstick is the exact logarithm rounded to double and
+    // then to float32.  (Rounding the exact logarithm to float32 in one step differs for one
+    // argument of them all, 0x1.827a74p-7, whose logarithm -0x1.1c2b1efffffffb1p+2 rounds to a
+    // double that lies exactly between two float32.)
+    if (argc > 2 && std::strcmp(argv[2], "all") == 0) {
+        std::atomic<long> flips{0}, count{0};
+        std::atomic<int> next{1};
+        std::vector<std::thread> workers;
+        for (int t = 0; t < 8; ++t)
+            workers.emplace_back([&] {
+                for (;;) {
+                    const int k = next.fetch_add(1);
+                    if (k > 53)
+                        break;
+                    long f = 0;
+                    for (uint32_t mant = 0; mant < (1u << 23); ++mant) {
+                        const float u = bm::bm_bits_to_float(((uint32_t)(127 - k) << 23) | mant);
+                        // rounded twice, to double and then to float32, as the callers do and as the
+                        // CPU restatement of the generators does
+                        f += (float)bm::bm_log_f32(u, &tab) != (float)(double)logl((long double)u);
+                    }
+                    flips += f;
+                    count += 1 << 23;
+                }
+            });
+        for (auto &w : workers)
+            w.join();
+        printf("log every float32 of [2^-53, 1): n=%ld float_flips=%ld\n", count.load(), flips.load());
     }
 
     // cosine: x = RN(RN(2 pi) * u) for u = k / 2^24 (float64 variant) and
