@@ -76,6 +76,31 @@ int main(int argc, char **argv)
         for (auto &w : workers)
             w.join();
         printf("log every float32 of [2^-53, 1): n=%ld float_flips=%ld\n", count.load(), flips.load());
+
+        // cosine of the float32 variant, the same way: the angle is RN32(RN32(2 pi) * u), the
+        // cosine is taken in double and rounded to float32; every u in [2^-53, 1)
+        std::atomic<long> cflips{0}, ccount{0};
+        next = 1;
+        workers.clear();
+        for (int t = 0; t < 8; ++t)
+            workers.emplace_back([&] {
+                for (;;) {
+                    const int k = next.fetch_add(1);
+                    if (k > 53)
+                        break;
+                    long f = 0;
+                    for (uint32_t mant = 0; mant < (1u << 23); ++mant) {
+                        const float u = bm::bm_bits_to_float(((uint32_t)(127 - k) << 23) | mant);
+                        const double x = (double)(6.283185307179586f * u);
+                        f += (float)bm::bm_cos_2pi(x, &tab) != (float)(double)cosl((long double)x);
+                    }
+                    cflips += f;
+                    ccount += 1 << 23;
+                }
+            });
+        for (auto &w : workers)
+            w.join();
+        printf("cos f32 every float32 of [2^-53, 1): n=%ld float_flips=%ld\n", ccount.load(), cflips.load());
     }
 
     // cosine: x = RN(RN(2 pi) * u) for u = k / 2^24 (float64 variant) and

@@ -18,7 +18,8 @@ def sweep(tmp_path_factory):
     subprocess.run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-pthread", "-I", CSRC,
                     os.path.join(HERE, "boxmuller_math_check.cpp"), "-o", exe], check=True)
     # every 7th mantissa: 1.2 M logarithms per binade and 2.4 M cosines per variant in ~1.5 s;
-    # "all": also the float32 rounding of the logarithm of every possible argument (~15 core-seconds)
+    # "all": also the float32 rounding of the logarithm and of the float32 variant's cosine for
+    # every possible argument (~40 core-seconds, 5 s on 8 cores)
     out = subprocess.run([exe, "7", "all"], check=True, capture_output=True, text=True).stdout
     return out
 
@@ -39,6 +40,15 @@ def test_logarithm_rounds_to_the_right_float32_for_every_possible_argument(sweep
     must be that of the exact logarithm rounded to double (long double carries 11 more bits
     than the double under test) for every one of them."""
     m = re.search(r"log every float32 of \[2\^-53, 1\): n=(\d+) float_flips=(\d+)", sweep)
+    assert int(m.group(1)) == 53 << 23 and int(m.group(2)) == 0
+
+
+def test_float32_cosine_rounds_to_the_right_float32_for_every_possible_argument(sweep):
+    """The float32 normal takes the cosine of RN32(RN32(2 pi) * u) in double and rounds it to
+    float32: the same yardstick, every u in [2^-53, 1).  Together with the logarithm above
+    (and a correctly rounded float32 square root and product) this makes the float32 normals
+    the bits of the CPU restatement for every pair of uniforms, not only for the sampled ones."""
+    m = re.search(r"cos f32 every float32 of \[2\^-53, 1\): n=(\d+) float_flips=(\d+)", sweep)
     assert int(m.group(1)) == 53 << 23 and int(m.group(2)) == 0
 
 
