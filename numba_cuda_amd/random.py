@@ -21,7 +21,7 @@ import math
 
 import numpy as np
 
-from numba_cuda_amd.cudadrv import devicearray, devices
+from numba_cuda_amd.cudadrv import devices
 from numba_cuda_amd.cudadrv import driver as _driver
 from numba_cuda_amd import api as _api
 

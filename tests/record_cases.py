@@ -2,8 +2,6 @@
 (numba_cuda/numba/cuda/tests/cudadrv/test_cuda_devicerecord.py), restated with the
 lines each case follows (numba type objects, :52-54, have no counterpart here).  Run
 on the fake library and on the GPU."""
-import ctypes
-
 import numpy as np
 
 from numba_cuda_amd.cudadrv.devicearray import DeviceRecord, auto_device, from_record_like

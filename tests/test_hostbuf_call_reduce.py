@@ -2,7 +2,6 @@
 Checked against a small native function compiled here that records its arguments."""
 
 import ctypes
-import os
 import shutil
 import subprocess
 

@@ -7,8 +7,6 @@ two calls in a row, the second on a smaller input, because the static array keep
 what the previous call left in it.
 """
 
-import ctypes
-
 import numpy as np
 import pytest
 
