@@ -267,10 +267,11 @@ def _workload(name, cuda):
                 s.synchronize()
 
         def extras():
-            """Where a call's time goes: the issuing loop alone (no waiting), and the same
+            """Where a call's time goes: the issuing loop alone (no waiting), the same
             4096 launches of this kernel issued through the bare native call with precomputed
             integer arguments - what the runtime's launch path costs per call, the floor
-            under any per-call interface."""
+            under any per-call interface on one host thread - and the whole step again with
+            the launches handed to a launching thread per stream."""
             from numba_cuda_amd.cudadrv import driver as drv
             from numba_cuda_amd.kernels import reduction
             cuda.synchronize()
@@ -293,8 +294,21 @@ def _workload(name, cuda):
                 call(*t)
             floor = time.perf_counter() - t0
             cuda.synchronize()
+            # the same step with a launching thread per stream (opt-in mode, off otherwise)
+            reduction.launch_threads(True)
+            try:
+                step(0)
+                cuda.synchronize()
+                t0 = time.perf_counter()
+                for k in range(3):
+                    step(k)
+                cuda.synchronize()
+                queued = (time.perf_counter() - t0) / (3 * rows)
+            finally:
+                reduction.launch_threads(False)
             return {"issue_us_per_call": round(issue / rows * 1e6, 3),
-                    "native_launch_us_per_call": round(floor / rows * 1e6, 3)}
+                    "native_launch_us_per_call": round(floor / rows * 1e6, 3),
+                    "launch_threads_us_per_call": round(queued * 1e6, 3)}
 
         return dict(desc="4096 x (65536 fp32) row sums round-robin over 4 streams, seed 3", dtype="f32",
                     algo_bytes=host.nbytes, units=rows, step=step, stream=streams[0], host=host,
@@ -422,8 +436,9 @@ def main():
         "pct_of_hbm_peak": head["pct_of_hbm_peak"], "units_per_s": head["units_per_s"],
         "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"],
     }
-    if "us_per_call" in head:
-        line["us_per_call"] = head["us_per_call"]
+    for key in head:
+        if key.endswith("us_per_call"):
+            line[key] = head[key]
 
     if args.workload is None and not args.no_others:
         # every other benchmark configuration, in this same process: fewer steps, and a CPU

@@ -184,6 +184,30 @@ int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, 
 int nbh_reduce_ordered(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                        void *scratch, size_t scratch_bytes, nbh_stream_t stream);
 
+/* Launching threads for loops of small reductions (no counterpart in the reference, whose
+ * Reduce.__call__ pays a kernel launch and an allocation on the calling thread,
+ * kernels/reduction.py:242-258).  The runtime's launch path costs 2.4 - 3.0 us per launch on
+ * one host thread and runs side by side from several.  After nbh_launch_threads(1),
+ * nbh_reduce_queued - same arguments and result as nbh_reduce; `init` is copied before the
+ * call returns - hands the launch to a thread that belongs to `stream` (made on first use,
+ * one per stream: the launches of a stream keep the order of the calls) and returns 0.
+ *   - Every entry point of this library that is given that stream first waits until its
+ *     queue has been launched; entry points that concern the whole device (a default stream,
+ *     synchronous copies, nbh_free, nbh_pool_free, nbh_device_synchronize ...) wait for all
+ *     queues.  Code OUTSIDE the library that was handed the stream does not: call
+ *     nbh_stream_synchronize first.  That is why the mode is off unless asked for.
+ *   - A launch that fails on the launching thread is reported by the next
+ *     nbh_stream_synchronize of the stream.
+ *   - The default streams (0, legacy, per-thread), and every call while the mode is off, go
+ *     straight to nbh_reduce.  nbh_launch_threads(0) waits for all queues and switches the
+ *     mode off; the threads sleep until their streams are destroyed.
+ *   - nbh_launch_threads_wait(stream) waits until what has been queued for `stream` (0: for
+ *     every stream) is in its stream, without waiting for the device. */
+int nbh_launch_threads(int enable);
+int nbh_launch_threads_wait(nbh_stream_t stream);
+int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
+                      void *scratch, size_t scratch_bytes, nbh_stream_t stream);
+
 /* nbh_reduce for callers that cannot allocate device memory: code under stream (graph)
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
  * in the reference (whose Reduce.__call__ allocates its partials on every call,

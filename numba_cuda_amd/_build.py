@@ -20,7 +20,7 @@ SRC_DIR = os.path.join(PKG_DIR, "csrc")
 INCLUDE_DIR = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libnbhip.so")
 
-SOURCES = ["runtime.hip", "hostcopy.hip", "pool.hip", "reduce.hip", "reduce_custom.hip", "transpose.hip", "assign.hip", "xoroshiro.hip"]
+SOURCES = ["runtime.hip", "hostcopy.hip", "pool.hip", "reduce.hip", "reduce_custom.hip", "launchq.hip", "transpose.hip", "assign.hip", "xoroshiro.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

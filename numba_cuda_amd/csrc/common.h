@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "nbhip.h"
 
 #define NBH_TRY(expr)                     \
@@ -17,7 +19,25 @@
 // the next synchronisation, as with any asynchronous HIP work.
 static inline int nbh_launch_status() { return (int)hipGetLastError(); }
 
-static inline hipStream_t nbh_hip_stream(nbh_stream_t s) { return (hipStream_t)s; }
+// Launching threads (launchq.hip, opt-in): a launch handed to a stream's thread is not in
+// the stream yet when the call returns, so whoever is about to put something else into that
+// stream waits for its queue first - here, where every entry point turns its stream argument
+// into the runtime's.  One relaxed load when the feature has never been switched on.
+extern std::atomic<int> nbh_queue_in_use;
+void nbh_queue_drain(nbh_stream_t stream);     // a default stream (0 included) stands for all streams
+void nbh_queue_forget(nbh_stream_t stream);    // before the stream is destroyed
+int nbh_queue_take_status(nbh_stream_t stream);
+static inline void nbh_queue_drain_all()
+{
+    if (nbh_queue_in_use.load(std::memory_order_relaxed))
+        nbh_queue_drain(nullptr);
+}
+static inline hipStream_t nbh_hip_stream(nbh_stream_t s)
+{
+    if (nbh_queue_in_use.load(std::memory_order_relaxed))
+        nbh_queue_drain(s);
+    return (hipStream_t)s;
+}
 
 // Number of compute units of the current device (cached per device).
 int nbh_cu_count();

@@ -182,6 +182,7 @@ int nbh_pool_free(void *ptr)
 {
     if (!ptr)
         return 0;
+    nbh_queue_drain_all();  // the events recorded below must come after every launch that names the block
     DevicePool *p = nullptr;
     if (int rc = current_pool(&p))
         return rc;

@@ -95,7 +95,11 @@ int nbh_device_attr(int dev, const char *name, int *value)
 }
 
 int nbh_mem_info(size_t *free_bytes, size_t *total_bytes) { return (int)hipMemGetInfo(free_bytes, total_bytes); }
-int nbh_device_synchronize(void) { return (int)hipDeviceSynchronize(); }
+int nbh_device_synchronize(void)
+{
+    nbh_queue_drain_all();
+    return (int)hipDeviceSynchronize();
+}
 
 // ---- memory ----------------------------------------------------------------
 
@@ -105,7 +109,11 @@ int nbh_malloc(void **dptr, size_t nbytes)
         return (int)hipErrorInvalidValue;
     return (int)hipMalloc(dptr, nbytes);
 }
-int nbh_free(void *dptr) { return (int)hipFree(dptr); }
+int nbh_free(void *dptr)
+{
+    nbh_queue_drain_all();  // a queued launch may still name this memory
+    return (int)hipFree(dptr);
+}
 int nbh_malloc_managed(void **ptr, size_t nbytes, int attach_global)
 {
     if (!ptr)
@@ -126,7 +134,11 @@ int nbh_host_alloc(void **hptr, size_t nbytes, unsigned flags)
         f |= hipHostMallocWriteCombined;
     return (int)hipHostMalloc(hptr, nbytes, f);
 }
-int nbh_host_free(void *hptr) { return (int)hipHostFree(hptr); }
+int nbh_host_free(void *hptr)
+{
+    nbh_queue_drain_all();
+    return (int)hipHostFree(hptr);
+}
 
 int nbh_host_register(void *hptr, size_t nbytes, unsigned flags)
 {
@@ -137,7 +149,11 @@ int nbh_host_register(void *hptr, size_t nbytes, unsigned flags)
         f |= hipHostRegisterMapped;
     return (int)hipHostRegister(hptr, nbytes, f);
 }
-int nbh_host_unregister(void *hptr) { return (int)hipHostUnregister(hptr); }
+int nbh_host_unregister(void *hptr)
+{
+    nbh_queue_drain_all();
+    return (int)hipHostUnregister(hptr);
+}
 int nbh_host_get_device_pointer(void **dptr, void *hptr) { return (int)hipHostGetDevicePointer(dptr, hptr, 0); }
 
 int nbh_mem_address_range(void **base, size_t *size, void *dptr)
@@ -188,7 +204,11 @@ int nbh_ipc_open(void **dptr, const void *handle, size_t nbytes)
     return (int)hipIpcOpenMemHandle(dptr, h, hipIpcMemLazyEnablePeerAccess);
 }
 
-int nbh_ipc_close(void *dptr) { return (int)hipIpcCloseMemHandle(dptr); }
+int nbh_ipc_close(void *dptr)
+{
+    nbh_queue_drain_all();
+    return (int)hipIpcCloseMemHandle(dptr);
+}
 
 static int copy(void *dst, const void *src, size_t nbytes, hipMemcpyKind kind, nbh_stream_t stream)
 {
@@ -270,10 +290,16 @@ int nbh_stream_create(nbh_stream_t *stream)
 }
 int nbh_stream_destroy(nbh_stream_t stream)
 {
+    nbh_queue_forget(stream);
     nbh_pool_forget_stream(nbh_hip_stream(stream));
     return (int)hipStreamDestroy(nbh_hip_stream(stream));
 }
-int nbh_stream_synchronize(nbh_stream_t stream) { return (int)hipStreamSynchronize(nbh_hip_stream(stream)); }
+int nbh_stream_synchronize(nbh_stream_t stream)
+{
+    const int rc = (int)hipStreamSynchronize(nbh_hip_stream(stream));
+    const int queued = nbh_queue_take_status(stream);  // a launch that a launching thread could not make
+    return rc ? rc : queued;
+}
 int nbh_stream_query(nbh_stream_t stream) { return (int)hipStreamQuery(nbh_hip_stream(stream)); }
 
 int nbh_stream_add_callback(nbh_stream_t stream, nbh_host_fn fn, void *user)

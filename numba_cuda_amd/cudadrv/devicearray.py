@@ -173,6 +173,11 @@ class DeviceNDArrayBase:
 
     @property
     def __cuda_array_interface__(self):
+        # whoever reads this is about to use the memory outside this package: launches still
+        # waiting in a launching thread's queue (kernels/reduction.py launch_threads) go first
+        lib = _driver.driver.lib if _driver.driver.is_initialized else None
+        if getattr(lib, "_launch_threads", False):
+            lib.nbh_launch_threads_wait(None)
         return {
             "shape": self.shape,
             "strides": None if is_contiguous(self) else tuple(self.strides),

@@ -411,13 +411,45 @@ _call_reduce = _driver._hostbuf.call_reduce
 _reduce_into = getattr(_driver._hostbuf, "reduce_into", lambda *args: NotImplemented)   # absent from an older build
 
 def _entry_address(lib):
-    """Address of the library's nbh_reduce for call_reduce, kept on the library object
-    (0: not a native function, e.g. a test double - call it the ordinary way)."""
+    """Address of the library's nbh_reduce (nbh_reduce_queued with launching threads) for
+    call_reduce and reduce_into, kept on the library object (0: not a native function, e.g. a
+    test double - call it the ordinary way)."""
     import ctypes
     try:
+        if _config.CUDA_REDUCE_LAUNCH_THREADS and not lib.nbh_launch_threads(1):
+            lib._launch_threads = True
+            return ctypes.cast(lib.nbh_reduce_queued, ctypes.c_void_p).value or 0
         return ctypes.cast(lib.nbh_reduce, ctypes.c_void_p).value or 0
     except (TypeError, ctypes.ArgumentError, AttributeError):
         return 0
+
+
+def launch_threads(enable=True):
+    """Hand the kernel launches of `Reduce(...)(arr, res=..., stream=s)` on streams made with
+    `cuda.stream()` to a launching thread per stream (True), or make them on the calling
+    thread again (False, the default; `NUMBA_CUDA_REDUCE_LAUNCH_THREADS=1` starts with True).
+    Not in the reference.  The runtime's launch path takes 2.4 - 3.0 us per launch on one host
+    thread and runs side by side from several, so a loop of small reductions over a few
+    streams gets through about twice as fast.  Everything this package does with such a
+    stream afterwards (copies, events, synchronize, other kernels) first waits until the
+    queued launches are in the stream, so results and ordering are those of the default mode.
+    Code outside the package that was handed the stream (`__cuda_array_interface__` consumers,
+    external-stream wrappers) cannot know about the queue: `stream.synchronize()` first."""
+    import ctypes
+    devices.get_context()                    # loads the library on the first call
+    lib = _driver.driver.lib
+    try:
+        entry = lib.nbh_reduce_queued if enable else lib.nbh_reduce
+        rc = lib.nbh_launch_threads(1 if enable else 0)
+    except AttributeError:
+        raise NotImplementedError("this build of the library has no launching threads") from None
+    if rc:
+        _driver.driver.check("nbh_launch_threads", rc)
+    lib._launch_threads = bool(enable)
+    try:
+        lib._reduce_entry = ctypes.cast(entry, ctypes.c_void_p).value or 0
+    except (TypeError, ctypes.ArgumentError):
+        lib._reduce_entry = 0
 
 
 _DTYPE_CODE = {np.dtype(name): code for name, code in _lib.DTYPE_CODES.items()}

@@ -9,6 +9,7 @@ import threading
 import time
 
 import numpy as np
+import pytest
 
 import numba_cuda_amd as cuda
 from numba_cuda_amd.cudadrv import driver as drv
@@ -170,3 +171,31 @@ def test_stream_callback_thunks_outlive_their_own_call(fake_gpu):
     assert seen == list(range(200))
     assert not drv._pending_thunks                  # every callback has run ...
     assert 0 < len(drv._finished_thunks) <= 65      # ... and its thunk was parked, not dropped, while running
+
+
+def test_launch_threads_switch_needs_a_library_that_has_them(monkeypatch):
+    """kernels/reduction.py launch_threads on a library without nbh_launch_threads (an older
+    build, a test double): says so instead of pretending."""
+    from numba_cuda_amd.kernels import reduction
+    from numba_cuda_amd.cudadrv import devices, driver as drv
+
+    class Bare:
+        pass
+
+    monkeypatch.setattr(devices, "get_context", lambda *a: None)
+    monkeypatch.setattr(drv.driver, "lib", Bare(), raising=False)
+    with pytest.raises(NotImplementedError):
+        reduction.launch_threads(True)
+
+
+def test_launch_threads_flag_is_read_from_the_environment(monkeypatch):
+    from numba_cuda_amd.core import config
+    assert config.CUDA_REDUCE_LAUNCH_THREADS == 0
+    monkeypatch.setenv("NUMBA_CUDA_REDUCE_LAUNCH_THREADS", "1")
+    config.reload_config()
+    try:
+        assert config.CUDA_REDUCE_LAUNCH_THREADS == 1
+    finally:
+        monkeypatch.delenv("NUMBA_CUDA_REDUCE_LAUNCH_THREADS")
+        config.reload_config()
+    assert config.CUDA_REDUCE_LAUNCH_THREADS == 0
