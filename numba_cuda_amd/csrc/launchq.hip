@@ -82,6 +82,10 @@ void run(Lane *lane)
     (void)hipSetDevice(lane->device);
     int idle = 0;
     for (;;) {
+        // asked to stop: whoever asks has waited for the queue first (nbh_queue_forget) or is
+        // ending the process, when nothing more may be launched
+        if (lane->stop.load(std::memory_order_acquire))
+            return;
         const uint64_t at = lane->issued.load(std::memory_order_relaxed);
         if (at != lane->pushed.load(std::memory_order_acquire)) {
             const Job &job = lane->ring[at % kRing];
@@ -95,8 +99,6 @@ void run(Lane *lane)
             idle = 0;
             continue;
         }
-        if (lane->stop.load(std::memory_order_acquire))
-            return;
         if (++idle < kSpins) {
             cpu_relax();
             continue;
@@ -194,8 +196,8 @@ bool is_default_stream(nbh_stream_t s)
     return s == nullptr || (hipStream_t)s == hipStreamLegacy || (hipStream_t)s == hipStreamPerThread;
 }
 
-// Joins the threads when the library is unloaded or the process ends (they are asleep or
-// polling an empty queue by then; nothing here calls into the runtime).
+// Joins the threads when the library is unloaded or the process ends.  Launches still queued
+// at that point are dropped (the runtime may be gone already); nothing here calls into it.
 struct AtExit {
     ~AtExit()
     {
@@ -271,11 +273,10 @@ int nbh_launch_threads(int enable)
         g_enabled.store(true, std::memory_order_release);
     } else {
         g_enabled.store(false, std::memory_order_release);
-        nbh_queue_drain(nullptr);  // the threads stay (asleep) until their streams go
-        // Nothing is queued any more and nothing will be: the entry points need not look.  (A
-        // call that read the switch just before it went off may still queue one launch; it
-        // raises the flag again itself.)
-        nbh_queue_in_use.store(0, std::memory_order_release);
+        // The threads stay (asleep) until their streams go, and nbh_queue_in_use stays up: a
+        // call that read the switch just before it went off may still queue one launch, and
+        // the entry points must go on looking for it.
+        nbh_queue_drain(nullptr);
     }
     return 0;
 }
@@ -313,7 +314,6 @@ int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, int64_t in_s
     job.out = out;
     job.scratch = scratch;
     job.scratch_bytes = scratch_bytes;
-    nbh_queue_in_use.store(1, std::memory_order_release);
     lane->pushed.store(at + 1);  // sequentially consistent: see run()
     rouse(lane);
     return 0;
