@@ -1,0 +1,85 @@
+// Host-side check of numba_cuda_amd/csrc/launchq.hip (the launching threads), no device needed:
+// a recording stand-in for nbh_reduce, six producers on six streams, waits for one queue and
+// for all, the mode switched off and on meanwhile, a stream destroyed and made again 300 times,
+// the error report.  Checks that every launch was made exactly once, in the order of the calls
+// of its stream, with its own arguments.  BURSTS=1 pauses the producers now and then so that
+// the launching threads fall asleep and have to be woken.  Built with the thread sanitizer and
+// run by tests/test_launchq_host.py.
+#include "common.h"
+#include <atomic>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <thread>
+#include <vector>
+extern "C" int nbh_launch_threads(int enable);
+extern "C" int nbh_launch_threads_wait(nbh_stream_t stream);
+extern "C" int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
+                                 void *scratch, size_t scratch_bytes, nbh_stream_t stream);
+static std::mutex g_m;
+static std::map<void *, std::vector<int64_t>> g_seen;   // per stream: the n of each launch, in order
+static std::atomic<long> g_calls{0};
+extern "C" int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
+                          void *scratch, size_t scratch_bytes, nbh_stream_t stream)
+{
+    (void)nbh_hip_stream(stream);   // what the real one does first
+    if (in_stride == 6) return 1;
+    {
+        std::lock_guard<std::mutex> h(g_m);
+        g_seen[stream].push_back(n);
+    }
+    *(int64_t *)out = n + *(const int32_t *)init;
+    g_calls++;
+    return 0;
+}
+void nbh_pool_note_stream(hipStream_t) {}
+void nbh_pool_forget_stream(hipStream_t) {}
+int main()
+{
+    nbh_launch_threads(1);
+    const int S = 6, N = 20000;
+    std::vector<void *> streams;
+    for (int s = 0; s < S; ++s) streams.push_back((void *)(uintptr_t)(0x1000 + 0x100 * s));
+    std::vector<std::vector<int64_t>> outs(S, std::vector<int64_t>(N, -1));
+    std::vector<std::thread> th;
+    int dummy_in = 0, scratch = 0;
+    for (int s = 0; s < S; ++s)
+        th.emplace_back([&, s] {
+            for (int i = 0; i < N; ++i) {
+                int32_t init = 7;
+                if (nbh_reduce_queued(0, 2, &dummy_in, i + 1, 4, &init, &outs[s][i], &scratch, 4, streams[s])) abort();
+                if (getenv("BURSTS") && i % 64 == 0) std::this_thread::sleep_for(std::chrono::microseconds(700));
+                if (i % 997 == 0) nbh_queue_drain(streams[s]);
+                if (i % 4999 == 0) nbh_queue_drain(nullptr);
+                if (s == 0 && i % 7001 == 0) { nbh_launch_threads(0); nbh_launch_threads(1); }
+            }
+        });
+    // a thread that keeps destroying and re-making a stream of its own
+    th.emplace_back([&] {
+        int64_t out = 0; int32_t init = 1;
+        for (int r = 0; r < 300; ++r) {
+            void *st = (void *)(uintptr_t)(0x9000 + 0x10 * (r % 3));
+            for (int i = 0; i < 20; ++i) nbh_reduce_queued(0, 2, &dummy_in, 5, 4, &init, &out, &scratch, 4, st);
+            nbh_queue_forget(st);
+            if (out != 6) { printf("bad out %ld\n", (long)out); abort(); }
+        }
+    });
+    for (auto &t : th) t.join();
+    nbh_queue_drain(nullptr);
+    for (int s = 0; s < S; ++s) {
+        for (int i = 0; i < N; ++i) if (outs[s][i] != i + 1 + 7) { printf("stream %d item %d: %ld\n", s, i, (long)outs[s][i]); return 1; }
+        const auto &v = g_seen[streams[s]];
+        if ((int)v.size() != N) { printf("stream %d saw %zu\n", s, v.size()); return 1; }
+        for (int i = 0; i < N; ++i) if (v[i] != i + 1) { printf("stream %d out of order at %d\n", s, i); return 1; }
+    }
+    // error report
+    int32_t init = 0; int64_t o = 0;
+    nbh_reduce_queued(0, 2, &dummy_in, 3, 6, &init, &o, &scratch, 4, streams[0]);
+    nbh_queue_drain(streams[0]);
+    if (nbh_queue_take_status(streams[0]) != 1 || nbh_queue_take_status(streams[0]) != 0) { printf("status\n"); return 1; }
+    for (void *st : streams) nbh_queue_forget(st);
+    printf("ok, %ld launches\n", g_calls.load());
+    return 0;
+}
