@@ -242,6 +242,89 @@ def test_normals_over_every_float32_mantissa_of_u1():
             np.testing.assert_array_equal(d.copy_to_host(), want_states)
 
 
+@pytest.mark.parametrize("binades", [range(1, 7), range(7, 13), range(13, 19), range(19, 25), range(25, 31),
+                                     range(31, 54)])
+def test_normals_for_every_value_the_first_uniform_can_take(binades):
+    """u1 = float32((draw >> 11) * 2^-53) is zero or one of 30 * 2^23 + 2^23 - 1 values: all 2^23
+    mantissas of the binades [2^-k, 2^-k+1) for k = 1 .. 30, and below that the multiples of
+    2^-53.  Every one of them goes through the device's logarithm and square root here (states
+    made so that the first draw is the chosen one; the second uniform is whatever the state
+    then yields): float32 normals must have the oracle's bits, float64 normals stay within
+    2 ulp."""
+    rng = np.random.default_rng(binades[0])
+    for k in binades:
+        if k <= 30:
+            mant = np.arange(1 << 23, dtype=np.uint64)
+            m53 = ((np.uint64(1) << np.uint64(23)) | mant) << np.uint64(30 - k)
+        else:
+            m53 = np.arange(1 << (53 - k), 1 << (54 - k), dtype=np.uint64)
+        n = m53.size
+        draw = m53 << np.uint64(11)
+        st = np.zeros(n, nrandom.xoroshiro128p_dtype)
+        st["s1"] = rng.integers(0, 2**63, n, dtype=np.uint64)
+        st["s0"] = draw - st["s1"]
+        for kind, dtype in (("normal_f32", np.float32), ("normal_f64", np.float64)):
+            d = cuda.to_device(st)
+            out = cuda.device_array(n, dtype)
+            nrandom.xoroshiro128p_fill(d, out, 1, nrandom.NORMAL)
+            want, _ = cref.fill(st, 1, kind)
+            got = out.copy_to_host()
+            if dtype is np.float32:
+                assert got.tobytes() == want.tobytes(), (k, kind, int((got != want).sum()))
+            else:
+                u = _ulps(got, want)
+                assert u.max() <= 2.0, (k, kind, float(u.max()))
+        _say("binade 2^-%d: %d values of u1" % (k, n))
+
+
+def _states_whose_second_draw_is(draw2, rng):
+    """States (s0, s1) whose SECOND 64-bit draw is `draw2`: pick the state after the first
+    step freely (s0' + s1' = draw2) and run the step backwards (random.py:62-93:
+    s1' = rotl(t, 36), s0' = rotl(s0, 55) ^ t ^ (t << 14) with t = s0 ^ s1)."""
+    u64 = np.uint64
+    def rotr(x, k):
+        return (x >> u64(k)) | (x << u64(64 - k))
+    s1n = rng.integers(0, 2**63, draw2.size, dtype=np.uint64)
+    s0n = draw2 - s1n
+    t = rotr(s1n, 36)
+    s0 = rotr(s0n ^ t ^ (t << u64(14)), 55)
+    st = np.zeros(draw2.size, nrandom.xoroshiro128p_dtype)
+    st["s0"] = s0
+    st["s1"] = t ^ s0
+    return st
+
+
+@pytest.mark.parametrize("binades", [range(1, 7), range(7, 13), range(13, 19), range(19, 25), range(25, 31),
+                                     range(31, 54)])
+def test_normals_for_every_value_the_second_uniform_can_take(binades):
+    """The same for u2, the argument of the cosine: states whose second draw is the chosen one
+    (the step run backwards), the first uniform whatever it then is."""
+    rng = np.random.default_rng(100 + binades[0])
+    for k in binades:
+        if k <= 30:
+            mant = np.arange(1 << 23, dtype=np.uint64)
+            m53 = ((np.uint64(1) << np.uint64(23)) | mant) << np.uint64(30 - k)
+        else:
+            m53 = np.arange(1 << (53 - k), 1 << (54 - k), dtype=np.uint64)
+        st = _states_whose_second_draw_is(m53 << np.uint64(11), rng)
+        if k == 1:   # the construction itself: the oracle's second uniform is the chosen one
+            u, _ = cref.fill(st[:1000], 2, "uniform_f64")
+            assert (u.reshape(-1, 2)[:, 1] == m53[:1000].astype(np.float64) * 2.0**-53).all()
+        n = st.size
+        for kind, dtype in (("normal_f32", np.float32), ("normal_f64", np.float64)):
+            d = cuda.to_device(st)
+            out = cuda.device_array(n, dtype)
+            nrandom.xoroshiro128p_fill(d, out, 1, nrandom.NORMAL)
+            want, _ = cref.fill(st, 1, kind)
+            got = out.copy_to_host()
+            if dtype is np.float32:
+                assert got.tobytes() == want.tobytes(), (k, kind, int((got != want).sum()))
+            else:
+                u = _ulps(got, want)
+                assert u.max() <= 2.0, (k, kind, float(u.max()))
+        _say("binade 2^-%d: %d values of u2" % (k, n))
+
+
 def test_scalar_functions_on_device_resident_states():
     """numba_cuda/numba/cuda/random.py:96-238 called from host code on the array
     create_xoroshiro128p_states returned: state and integer / uniform bits exact against
