@@ -228,7 +228,7 @@ def _workload(name, cuda):
                 nrandom.xoroshiro128p_fill(states, out, 64, nrandom.UNIFORM, stream)
             return dict(desc="xoroshiro128p 2^24 generators x 64 uniform float32", dtype="u64",
                         algo_bytes=4 * n * 64 + 32 * n, units=n * 64, step=step, stream=stream, host=None,
-                        kernel="fill_kernel<UniformF32>", keep=(states, out))
+                        kernel="fill_regs_kernel<UniformF32>", keep=(states, out))
         if name == "rng_normal_f64":
             out = cuda.device_array(n * 16, np.float64)
 

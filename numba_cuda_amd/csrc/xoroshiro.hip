@@ -587,6 +587,100 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
     }
 }
 
+// Runs of whole 256-byte pieces on 128-byte lines, cheap generators.  The kernel above parks a
+// round of every lane in LDS - 17 KB per wavefront with two lines per round, which leaves room
+// for two wavefronts per SIMD, too few to keep the vector ALU busy while some of them wait for
+// their stores.  Here a lane draws its 256 bytes into REGISTERS, and the wavefront hands them
+// over sixteen generators at a time through 4 KB of LDS: the sixteen lanes of a quarter park
+// their runs, all 64 lanes read them back as (generator, packet) and store - four store
+// instructions of 1 KiB, each over four whole runs, so a wavefront still writes its 16 KiB as
+// one piece.  Occupancy is then bounded by registers (four wavefronts per SIMD), and which XCD
+// writes what starts to matter: with each XCD writing 256 KiB in a row (`runs` workgroups)
+// 2^24 generators x 64 float32 take 710 - 728 us against 770 with every eighth workgroup's 64 KiB
+// and 745 - 757 for the kernel above (where the order makes no difference).  Alone, the stores
+// of this pattern take 675 us (805 without the runs) and the generation 587 us.
+// Consecutive workgroups are started on different XCDs (workgroup b on XCD b % 8).  Within
+// every whole group of 8 * runs consecutive workgroups this hands XCD k the pieces k * runs ...
+// k * runs + runs - 1, so that an XCD writes `runs` workgroups' worth in a row; the workgroups
+// past the last whole group keep their own piece.
+__device__ __forceinline__ int64_t piece_of_block(int64_t block, int64_t grid, int runs)
+{
+    const int64_t span = 8 * (int64_t)runs;
+    if (runs <= 1 || block >= grid / span * span)
+        return block;
+    const int64_t r = block % span;
+    return block - r + (r % 8) * runs + r / 8;
+}
+template <typename Gen>
+__global__ __launch_bounds__(kFillBlock) void fill_regs_kernel(uint64_t *__restrict__ states, int64_t n,
+                                                               typename Gen::value_type *__restrict__ out,
+                                                               int64_t count, int runs)
+{
+    static_assert(!Gen::kHeavy, "for the generators that are bound by their stores");
+    using VT = typename Gen::value_type;
+    constexpr int PER = 16 / (int)sizeof(VT);     // values per 16-byte packet
+    constexpr int ROUND = 256 / (int)sizeof(VT);  // values per generator and round
+    constexpr int PK = ROUND / PER;               // packets per generator and round: 16
+    constexpr int PITCH = ROUND + PER;            // 272-byte rows
+    __shared__ __attribute__((aligned(16))) VT park_all[kFillBlock / 64][16][PITCH];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    VT(*park)[PITCH] = park_all[wave];
+    const int64_t t0 = (piece_of_block(blockIdx.x, gridDim.x, runs) * (kFillBlock / 64) + wave) * 64;
+    if (t0 >= n)
+        return;
+    const int64_t t = t0 + lane;
+    const bool live = t < n;
+    typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+    uint64_t s0 = 0, s1 = 0;
+    if (live) {
+        u64x2 v = *reinterpret_cast<const u64x2 *>(states + 2 * t);
+        s0 = v.x;
+        s1 = v.y;
+    }
+    const int lanes_here = (n - t0 > 64) ? 64 : (int)(n - t0);
+    VT *__restrict__ base = out + t0 * count;
+    const int quarter = lane >> 4, packet = lane & 15;
+
+    for (int64_t i0 = 0; i0 < count; i0 += ROUND) {   // count is a multiple of ROUND (the host's check)
+        union {
+            VT val[ROUND];
+            u32x4 pk[PK];
+        } mine;
+#pragma unroll
+        for (int j = 0; j < ROUND; ++j)
+            mine.val[j] = Gen::draw(s0, s1, nullptr);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (quarter == q) {
+#pragma unroll
+                for (int k = 0; k < PK; ++k)
+                    *reinterpret_cast<u32x4 *>(&park[lane & 15][k * PER]) = mine.pk[k];
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = 4 * i + quarter;          // a store instruction covers rows 4 i ... 4 i + 3
+                const int gen = 16 * q + row;
+                if (gen < lanes_here) {
+                    u32x4 v = *reinterpret_cast<const u32x4 *>(&park[row][packet * PER]);
+                    nbh_store16<(int)sizeof(VT), true>(base + (int64_t)gen * count + i0 + packet * PER, v);
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    }
+    if (live) {
+        u64x2 v = {s0, s1};
+        *reinterpret_cast<u64x2 *>(states + 2 * t) = v;
+    }
+}
+
 // Runs that do not start on 128-byte lines (count * itemsize not a multiple of 128, or
 // an unaligned array) and are longer than a line.  Cutting the rounds where the runs
 // start makes every store of the kernel above straddle two lines.  Here the rounds of
@@ -795,6 +889,19 @@ struct RingLaunch<Gen, true> {
     static void go(dim3, hipStream_t, uint64_t *, int64_t, typename Gen::value_type *, int64_t) {}
 };
 
+template <typename Gen, bool Heavy = Gen::kHeavy>
+struct FillRegs {
+    static void go(dim3 grid, hipStream_t s, uint64_t *states, int64_t n, typename Gen::value_type *out, int64_t count,
+                   int runs)
+    {
+        hipLaunchKernelGGL((fill_regs_kernel<Gen>), grid, dim3(kFillBlock), 0, s, states, n, out, count, runs);
+    }
+};
+template <typename Gen>
+struct FillRegs<Gen, true> {
+    static void go(dim3, hipStream_t, uint64_t *, int64_t, typename Gen::value_type *, int64_t, int) {}
+};
+
 template <typename Gen>
 int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t stream)
 {
@@ -827,6 +934,16 @@ int launch_fill(void *states, int64_t n, void *out, int64_t count, nbh_stream_t 
     if (on_lines && lines == 4)
         hipLaunchKernelGGL((fill_kernel<Gen, true, 4>), dim3((unsigned)grid), dim3(kFillBlock), 0,
                            nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);
+    else if (on_lines && lines == 2 && (run_bytes == 256 || run_bytes == 512)) {
+        // (measured, 2^22 generators, this kernel against the one above: 64 float32 194 -> 183 us,
+        // 128 float32 436 -> 422, 32 float64 194 -> 183, 64 float64 the same; longer runs lose:
+        // 192 float32 576 -> 598, 256 float32 780 -> 802)
+        // a workgroup writes kFillBlock runs in a row; XCDs take turns after 256 KiB
+        int runs = 1;
+        while ((uint64_t)runs * kFillBlock * run_bytes < (256u << 10))
+            runs *= 2;
+        FillRegs<Gen>::go(dim3((unsigned)grid), nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, runs);
+    }
     else if (on_lines && lines == 2)
         hipLaunchKernelGGL((fill_kernel<Gen, true, 2>), dim3((unsigned)grid), dim3(kFillBlock), 0,
                            nbh_hip_stream(stream), (uint64_t *)states, n, (VT *)out, count, log_table);

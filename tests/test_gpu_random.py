@@ -71,9 +71,10 @@ def _ulps(got, want):
         np.spacing(np.abs(want[fin])).astype(np.float64)
 
 
-@pytest.mark.parametrize("n", [1, 64, 257, 5000])
+@pytest.mark.parametrize("n", [1, 64, 257, 5000, 70001])
 @pytest.mark.parametrize("kind,count", [("uniform_f32", 64), ("uniform_f32", 1), ("uniform_f32", 33),
-                                        ("uniform_f64", 7), ("uniform_f64", 40),
+                                        ("uniform_f32", 128), ("uniform_f32", 192), ("uniform_f32", 96),
+                                        ("uniform_f64", 7), ("uniform_f64", 40), ("uniform_f64", 32), ("uniform_f64", 96),
                                         ("normal_f32", 33), ("normal_f64", 16)])
 def test_fill_against_oracle(n, kind, count):
     _say("fill", kind, n, count)
