@@ -447,6 +447,11 @@ def main():
         for other in OTHER_WORKLOADS:
             _release_device_memory(cuda)
             steps, warmup = (10, 2) if other == "batched_reduce" else (min(args.steps, 50), min(args.warmup, 5))
+            if other in ("rng_uniform_f32", "rng_normal_f64"):
+                # millisecond-long, arithmetic-heavy launches: the device's power management lets the
+                # first three run fast, throttles the next ones by up to 40 % and takes some fifty
+                # launches to settle (profiles/xoroshiro_fill_and_init_2p24.txt); sixty untimed ones first
+                warmup = max(warmup, 60)
             print("bench: %s ..." % other, file=sys.stderr, flush=True)
             others.append(measure(cuda, other, steps, warmup, 0 if args.no_cpu_baseline else 2.0))
         line["others"] = others
