@@ -117,8 +117,18 @@ __global__ __launch_bounds__(64 * Shape::WR * Shape::WC) void transpose_packets(
     constexpr int TR = WT * WR * REP, TC = WT * WC;
 
     // consecutive workgroups go down the input rows = along the output rows
-    const int64_t tile_c = (int64_t)blockIdx.x / tiles_r;
+    int64_t tile_c = (int64_t)blockIdx.x / tiles_r;
     const int64_t tile_r = (int64_t)blockIdx.x % tiles_r;
+    if (E == 2) {
+        // 2-byte items: the column bands are walked in two passes, even bands first, then odd
+        // ones, so that bands side by side are not in flight together.  Measured, bands in
+        // order -> two passes, us: 8192 x 32768 191.3 -> 188.1, 32768 x 8192 216.8 -> 209.9,
+        // 16384^2 214.9 -> 211.6, 8192^2 51.1 -> 49.3.  (4- and 8-byte items: 8192^2 float32
+        // 96.3 -> 93.0, 12288^2 220.9 -> 213.8, but 16384^2 353 -> 364 and float64
+        // 8192 x 16384 353 -> 373: no rule that holds there, so they keep the plain order.)
+        const int64_t tiles_c = (int64_t)gridDim.x / tiles_r, half = (tiles_c + 1) / 2;
+        tile_c = tile_c < half ? tile_c * 2 : (tile_c - half) * 2 + 1;
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wr = wave / WC, wc = wave % WC;
     const int cx = lane & 7, ry = lane >> 3;
@@ -141,28 +151,34 @@ __global__ __launch_bounds__(64 * Shape::WR * Shape::WC) void transpose_packets(
 // 128-byte piece a wavefront stores would straddle two lines (measured: float32,
 // 16388 rows, 4.1 TB/s against 5.4 TB/s when only the INPUT rows straddle).  Here a
 // workgroup walks down a strip of the input, TR rows at a time, through a ring of
-// RING = TR + L rows in LDS (L = items per line), and for every output row c it
-// writes the items r in [lo(c), hi(c)), both ends rounded down to the nearest r at
-// which output row c crosses a line boundary.  Eight lanes write one line as eight
-// aligned 16-byte packets, non-temporally, so every store instruction covers eight
-// whole lines.  What lies below hi(c) stays in the ring for the next step, so nothing
-// is read twice except the L rows above the start of a strip.  The ring's row pitch
-// (TC + PAD items) spreads the column reads of one store instruction over the banks.
+// RING = TR + S rows in LDS, and for every output row c it writes the items r in
+// [lo(c), hi(c)), both ends rounded down to the nearest r at which output row c crosses
+// a SECTOR boundary (S items).  Eight lanes write one line as eight aligned 16-byte
+// packets, non-temporally, so every store instruction covers whole lines except where
+// a tile's part of an output row begins or ends inside a line: there the lanes outside
+// [lo, hi) stay idle and the rest of the line comes from the tile above or below.  What
+// lies below hi(c) stays in the ring for the next step, so nothing is read twice except
+// the S rows above the start of a strip.  Sectors of 32 bytes are what the memory takes
+// as whole writes; with whole lines as the unit (S = items per line) every tile reads
+// the 16 float64 rows above it a second time - 14 % more input traffic for a 112-row
+// tile, against 3 % with 4-row sectors.  The ring's row pitch (TC + PAD items) spreads
+// the column reads of one store instruction over the banks.
 // Measured: float64 12345 x 6789 4.0 -> 5.1 TB/s, float32 16388 x 16384 4.1 -> 5.0.
 // One-byte items stay with the packet kernel: gathering 16 single bytes from the ring
 // per store costs more than the straddling does (2.5 against 3.2 TB/s).
 // Shape of the ring kernel.  RING (a power of two) rows of TC columns, THREADS lanes,
-// STEPS steps of TR = RING - L rows per workgroup.
-template <int E_, int RING_, int TC_, int PAD_, int THREADS_, int STEPS_> struct RingCfg {
+// STEPS steps of TR = RING - SECTOR / E rows per workgroup.
+template <int E_, int RING_, int TC_, int PAD_, int THREADS_, int STEPS_, int SECTOR_ = 128> struct RingCfg {
     static constexpr int E = E_, RING = RING_, TC = TC_, PAD = PAD_, THREADS = THREADS_, STEPS = STEPS_;
+    static constexpr int SECTOR = SECTOR_ < E_ * 2 ? E_ * 2 : SECTOR_;  // at least two items: 16-byte items
 };
 // Measured on MI355X (TB/s of algorithmic traffic, ring 64 rows x 8 steps -> these shapes):
 // float64 12345 x 6789 5.07 -> 5.44, float32 16388 x 16384 5.10 -> 5.75, 16385^2 5.09 -> 5.32,
 // int16 8193 x 32769 4.40 -> 5.04, 16-byte items 8193^2 5.18 -> 5.86.  Tall tiles win (long
 // runs of every output row are written by one workgroup at one time) and so do short
 // strips: with one step per workgroup there are more, shorter workgroups in flight and
-// the L rows above a strip, read a second time, cost less than the lost overlap did.
-// 2-byte items: 256 x 64 in two steps with 256 threads -> one step of 192 rows with 512
+// the rows above a strip, read a second time, cost less than the lost overlap did.
+// 2-byte items: 256 x 64 in two steps with 256 threads -> one step with 512
 // threads and the unguarded interior path: 8193 x 32769 214 -> 206 us, 30001 x 7001 195 -> 183.
 template <int E> struct ShearOf;
 template <> struct ShearOf<2> { using type = RingCfg<2, 256, 64, 8, 512, 1>; };
@@ -181,11 +197,12 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
     using Item = typename ItemOf<E>::type;
     constexpr int V = 16 / E;    // items per packet
     constexpr int L = 128 / E;   // items per cache line
+    constexpr int S = Cfg::SECTOR / E;  // items per sector: where a tile's part of an output row begins and ends
     constexpr int RING = Cfg::RING, TC = Cfg::TC, kThr = Cfg::THREADS;
-    constexpr int TR = RING - L;
+    constexpr int TR = RING - S;
     constexpr int PPR = TC / V;     // packets per tile row
-    constexpr int NL = TR / L + 2;  // lines of one output row a step can touch, at most
-    static_assert((RING & (RING - 1)) == 0 && TR > 0, "ring depth");
+    constexpr int NL = RING / L + 1;  // lines of one output row a step can touch, at most
+    static_assert((RING & (RING - 1)) == 0 && TR > 0 && S % V == 0 && L % S == 0 && RING % L == 0, "ring depth");
     __shared__ Item ring[RING][TC + Cfg::PAD];
 
     const int tid = threadIdx.x;
@@ -228,23 +245,24 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
 
     // Tiles of a one-step configuration that lie wholly inside the matrix (`lean`: the host
     // asks for this path where it was measured to win): nothing needs a guard, so
-    // the tile and the L rows above it arrive with ONE round of loads (the general path
-    // below waits for the L rows before it asks for the rest), and every thread then writes
-    // TR / L lines of one output row, 128 bytes apart, all read from LDS before the first
-    // store.  Measured, general path -> this one: float64 12345 x 6789 246 -> 234 us (with
-    // the padded order), float32 16100^2 391 -> 369, 12345 x 13578 259 -> 239.  With input
+    // the tile and the S rows above it arrive with ONE round of loads (the general path
+    // below waits for those rows before it asks for the rest), and every thread then writes
+    // its 16-byte piece of every line of one output row, 128 bytes apart, all read from
+    // LDS before the first store.  Measured with whole lines as the sector, general path ->
+    // this one: float64 12345 x 6789 246 -> 234 us (with the padded order), float32 16100^2
+    // 391 -> 369, 12345 x 13578 259 -> 239.  With input
     // rows ON the grid it is slower for 4- and 8-byte items (float32 16388 x 16384 374 -> 391,
     // float64 4099 x 20000 229 -> 243) and for 16-byte items always (8193^2 366 -> 401):
     // those keep the general path.  2-byte items gain either way (8193 x 32769 214 -> 206,
     // 10001 x 12001 88 -> 75, input rows on the grid 8193 x 32768 206 -> 205).
     if constexpr (Cfg::STEPS == 1 && E < 16) {
-        if (lean && strip_begin >= L && strip_begin + TR < rows && C0 + TC <= cols) {
+        if (lean && strip_begin >= S && strip_begin + TR < rows && C0 + TC <= cols) {
             constexpr int RPS = kThr / PPR;      // tile rows one round of the workgroup loads
             constexpr int NPF = RING * PPR / kThr;
-            constexpr int NLF = TR / L;          // whole lines per output row
+            constexpr int NLF = (RING + L - 2 * S + L - 1) / L;  // line slots of one output row
             static_assert(RING * PPR % kThr == 0 && kThr % PPR == 0, "whole rounds of loads");
-            static_assert(kThr / 8 == TC && TR % L == 0, "eight lanes per output row");
-            const int64_t A = strip_begin - L;
+            static_assert(kThr / 8 == TC, "eight lanes per output row");
+            const int64_t A = strip_begin - S;
             const int lr0 = tid / PPR, pc = tid % PPR;
             const char *src = in + (A + lr0) * in_s0 + (C0 + (int64_t)pc * V) * E;
             u32x4 got[NPF];
@@ -258,18 +276,26 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
             const int lc = tid >> 3, sub = tid & 7;
             char *row = out + (C0 + lc) * out_s0;
             const int phase = (int)(((uintptr_t)row % 128) / E);
-            const int64_t lo = strip_begin - (phase + strip_begin) % L;  // in (strip_begin - L, strip_begin]
-            const int d = (int)(lo - A) + sub * V;                         // tile row of this lane's first item
+            // this tile's part of the output row: [lo, lo + TR), lo in (strip_begin - S, strip_begin]
+            const int lo_t = S - (int)((phase + strip_begin) % S);   // tile row of item lo, in [1, S]
+            const int first_t = lo_t - (int)((phase + A + lo_t) % L); // tile row at which lo's line begins (may be < 0)
             Pack p[NLF];
 #pragma unroll
-            for (int i = 0; i < NLF; ++i)
+            for (int i = 0; i < NLF; ++i) {
+                const int d = first_t + i * L + sub * V;  // tile row of this lane's first item
+                if (d >= lo_t && d < lo_t + TR) {
 #pragma unroll
-                for (int j = 0; j < V; ++j)
-                    p[i].it[j] = ring[d + i * L + j][lc];
-            char *dst = row + (lo + sub * V) * E;  // 16-byte aligned: lo starts a line
+                    for (int j = 0; j < V; ++j)
+                        p[i].it[j] = ring[d + j][lc];
+                }
+            }
+            char *dst = row + (A + first_t + sub * V) * E;  // 16-byte aligned: first_t starts a line
 #pragma unroll
-            for (int i = 0; i < NLF; ++i)
-                __builtin_nontemporal_store(p[i].pk, reinterpret_cast<u32x4 *>(dst + i * 128));
+            for (int i = 0; i < NLF; ++i) {
+                const int d = first_t + i * L + sub * V;
+                if (d >= lo_t && d < lo_t + TR)
+                    __builtin_nontemporal_store(p[i].pk, reinterpret_cast<u32x4 *>(dst + i * 128));
+            }
             return;
         }
     }
@@ -312,8 +338,8 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
         }
     };
 
-    fetch(strip_begin - L, strip_begin);  // what the first step needs from above
-    park(strip_begin - L, strip_begin);
+    fetch(strip_begin - S, strip_begin);  // what the first step needs from above
+    park(strip_begin - S, strip_begin);
     int64_t R0 = strip_begin;
     int64_t step_end = (R0 + TR < strip_end) ? R0 + TR : strip_end;
     fetch(R0, step_end);
@@ -333,21 +359,23 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
                 continue;
             char *row = out + c * out_s0;
             const int64_t phase = (int64_t)(((uintptr_t)row % 128) / E);  // line offset of item 0, in items
-            const int64_t hi = (step_end == rows) ? rows : step_end - (phase + step_end) % L;
-            const int64_t line = R0 - (phase + R0) % L + (int64_t)k * L;  // first item of this line
+            // this step's part of the output row: [lo, hi), both on sector boundaries of the row
+            const int64_t lo = (R0 == 0) ? 0 : R0 - (phase + R0) % S;
+            const int64_t hi = (step_end == rows) ? rows : step_end - (phase + step_end) % S;
+            const int64_t line = lo - (phase + lo) % L + (int64_t)k * L;  // first item of this line (below 0 in row 0's first line)
             if (line >= hi)
                 continue;
             const int64_t r = line + (tid & 7) * V;
             Pack p;
-            if (line >= 0 && line + L <= hi) {
+            if (r >= lo && r + V <= hi) {
 #pragma unroll
                 for (int j = 0; j < V; ++j)
                     p.it[j] = ring[(r + j) & (RING - 1)][lc];
                 u32x4 *dst = reinterpret_cast<u32x4 *>(row + r * E);  // 16-byte aligned: the line is
                 __builtin_nontemporal_store(p.pk, dst);
-            } else {  // first line of the matrix or last line of it
+            } else {  // where the matrix begins or ends inside a packet
                 for (int j = 0; j < V; ++j)
-                    if (r + j >= 0 && r + j < hi)
+                    if (r + j >= lo && r + j < hi)
                         *reinterpret_cast<Item *>(row + (r + j) * E) = ring[(r + j) & (RING - 1)][lc];
             }
         }
@@ -505,7 +533,7 @@ int launch_sheared_cfg(const void *in, void *out, int64_t rows, int64_t cols, in
                        hipStream_t stream)
 {
     constexpr int E = Cfg::E;
-    constexpr int TR = Cfg::RING - 128 / E;
+    constexpr int TR = Cfg::RING - Cfg::SECTOR / E;
     const int64_t strips_r = (rows + (int64_t)Cfg::STEPS * TR - 1) / ((int64_t)Cfg::STEPS * TR);
     const int64_t tiles_c = (cols + Cfg::TC - 1) / Cfg::TC;
     const bool ragged_in = (((uint64_t)(uintptr_t)in | (uint64_t)in_s0) % 128) != 0;
