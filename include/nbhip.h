@@ -200,7 +200,9 @@ int nbh_reduce_ordered(int op, int dtype, const void *in, int64_t n, int64_t in_
  *     nbh_stream_synchronize of the stream.
  *   - The default streams (0, legacy, per-thread), and every call while the mode is off, go
  *     straight to nbh_reduce.  nbh_launch_threads(0) waits for all queues and switches the
- *     mode off; the threads sleep until their streams are destroyed.
+ *     mode off; the threads sleep until their streams are destroyed.  nbh_launch_threads(-1)
+ *     does the same and then joins every thread: for the end of a process, before the GPU
+ *     runtime's own exit handlers run.  A forked child starts with the mode off and no queues.
  *   - nbh_launch_threads_wait(stream) waits until what has been queued for `stream` (0: for
  *     every stream) is in its stream, without waiting for the device. */
 int nbh_launch_threads(int enable);
@@ -220,9 +222,15 @@ int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, int64_t in_s
  * outside stream capture.
  *   - n above NBH_REDUCE_NOALLOC_MAX_ITEMS is refused with hipErrorInvalidValue before
  *     anything is launched
- *   - every call on a device shares that device's array: calls that may overlap in time
- *     (different streams, different host threads) race and give wrong results; callers
- *     that need overlap bring one scratch buffer per stream to nbh_reduce instead
+ *   - every call on a device shares that device's array: calls that overlap in time would
+ *     race.  A call on another stream than the previous call's, made while that call's
+ *     kernel has not finished, is refused with hipErrorNotReady (an event query, no wait);
+ *     calls on one stream, and calls involving the null stream, are ordered by the stream.
+ *     Under stream capture the check is left out (nothing runs then): replays of graphs
+ *     that hold such calls must not overlap.  Callers that need overlap bring one scratch
+ *     buffer per stream to nbh_reduce instead
+ *   - a call that fails after its launch marks the array; the next call clears the ticket
+ *     with a one-workgroup kernel on its stream before it starts
  *   - the array starts zeroed and each call leaves its ticket at zero again; the partials
  *     keep the last call's values and are overwritten before they are read */
 #define NBH_REDUCE_NOALLOC_MAX_ITEMS ((int64_t)1 << 36)

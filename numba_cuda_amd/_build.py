@@ -58,12 +58,14 @@ def build_hostbuf(verbose=False):
     cc = os.environ.get("CC") or shutil.which("gcc") or shutil.which("cc")
     if not cc:
         raise RuntimeError("no C compiler found for numba_cuda_amd/cext/hostbuf.c (set CC)")
-    tmp = HOSTBUF_PATH + ".tmp"
+    tmp = "%s.tmp.%d" % (HOSTBUF_PATH, os.getpid())     # importers in several processes may build at once
     cmd = [cc, "-O2", "-Wall", "-shared", "-fPIC", "-I", sysconfig.get_paths()["include"], HOSTBUF_SRC, "-o", tmp]
     if verbose:
         print(" ".join(cmd))
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
+        if os.path.exists(tmp):
+            os.unlink(tmp)
         raise RuntimeError("building _hostbuf failed:\n" + proc.stdout)
     os.replace(tmp, HOSTBUF_PATH)
     return HOSTBUF_PATH
@@ -110,13 +112,41 @@ def build(verbose=False, only=None):
     with ThreadPoolExecutor(max_workers=workers) as pool:
         for _ in pool.map(lambda cmd: _run(cmd, verbose), jobs):
             pass
-    tmp = LIB_PATH + ".tmp"
+    tmp = "%s.tmp.%d" % (LIB_PATH, os.getpid())
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", tmp], verbose)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
+
+
+RELEASE_PUBLISH_LIB = os.path.join(PKG_DIR, "libnbhip_release_publish.so")
+
+
+def build_release_publish(verbose=False):
+    """A second library whose reduction kernels publish their partials the by-the-book way
+    (csrc/reduce.hip built with -DNBH_REDUCE_RELEASE_PUBLISH=1: ordinary stores, then a release
+    at agent scope).  Not used by the package: the GPU tests run it beside libnbhip.so to keep
+    that path compiling and bit-equal.  Reuses the other object files of build()."""
+    hipcc = find_hipcc()
+    obj_dir = os.path.join(PKG_DIR, "_obj")
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    objects = []
+    for src in SOURCES:
+        obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+        if src == "reduce.hip":
+            obj = os.path.join(obj_dir, "reduce.release_publish.o")
+            _run([hipcc] + compile_flags + ["-DNBH_REDUCE_RELEASE_PUBLISH=1", "-I", INCLUDE_DIR, "-I", SRC_DIR, "-c",
+                                            os.path.join(SRC_DIR, src), "-o", obj], verbose)
+        elif not os.path.exists(obj):
+            raise RuntimeError("build() first: %s is missing" % obj)
+        objects.append(obj)
+    tmp = "%s.tmp.%d" % (RELEASE_PUBLISH_LIB, os.getpid())
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", tmp], verbose)
+    os.replace(tmp, RELEASE_PUBLISH_LIB)
+    return RELEASE_PUBLISH_LIB
 
 
 if __name__ == "__main__":
     print(build_hostbuf(verbose="-v" in sys.argv))
     names = [a for a in sys.argv[1:] if a.endswith(".hip")]
     print(build(verbose="-v" in sys.argv, only=names or None))
+    print(build_release_publish(verbose="-v" in sys.argv))

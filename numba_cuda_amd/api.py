@@ -48,6 +48,11 @@ def to_device(obj, stream=0, copy=True, to=None):
     return devicearray.auto_device(obj, stream=stream, copy=copy, user_explicit=True)[0]
 
 
+def _auto_device(ary, stream=0, copy=True):
+    """(device array, was a copy made): what kernel launchers use for their arguments."""
+    return devicearray.auto_device(ary, stream=stream, copy=copy)
+
+
 def _layout_like(ary):
     """(strides, order) that give a compact array with `ary`'s shape and axis
     ordering; strides is None when plain C / F order already does."""

@@ -15,6 +15,12 @@
 // __cuda_array_interface__ or an external-stream wrapper) does not know about the queue; a
 // caller who mixes the two must call nbh_stream_synchronize or nbh_queue_drain first.  Hence
 // opt-in.  The default streams (0, legacy, per-thread) are never queued.
+// A forked child has none of the threads and may hold a copy of a locked lock: a
+// pthread_atfork handler empties the child's list of queues and switches the feature off
+// there, so that no entry point waits for a thread that does not exist.  At the end of a
+// process nbh_launch_threads(-1) (called by the Python layer from an exit hook, before the
+// runtime's own exit handlers run) launches what is queued and joins the threads; the static
+// destructor below only catches what was never stopped that way.
 #include "common.h"
 
 #include <atomic>
@@ -24,6 +30,9 @@
 #include <thread>
 #include <vector>
 
+#include <new>
+
+#include <pthread.h>
 #include <unistd.h>
 
 std::atomic<int> nbh_queue_in_use{0};
@@ -167,6 +176,8 @@ Lane *lane_of(nbh_stream_t stream, bool make)
 
 void wait_launched(Lane *lane)
 {
+    if (lane->owner != getpid())
+        return;  // a forked child: the thread that would launch them does not exist here
     const uint64_t upto = lane->pushed.load(std::memory_order_acquire);
     if (lane->issued.load(std::memory_order_acquire) >= upto)
         return;
@@ -189,6 +200,38 @@ void retire(Lane *lane)
     if (lane->worker.joinable())
         lane->worker.join();
     delete lane;
+}
+
+// In the child of a fork: forget the queues (their threads are the parent's), take a fresh lock
+// in place of one that may have been copied while held, switch the feature off.
+void after_fork_in_child()
+{
+    new (&g_lock) std::mutex;
+    new (&g_lanes) std::vector<Lane *>;   // the lanes are left behind: their threads and locks belong to the parent
+    g_enabled.store(false, std::memory_order_release);
+    nbh_queue_in_use.store(0, std::memory_order_release);
+    g_generation.fetch_add(1, std::memory_order_release);
+}
+
+void register_fork_handler()
+{
+    static std::once_flag once;
+    std::call_once(once, [] { pthread_atfork(nullptr, nullptr, after_fork_in_child); });
+}
+
+// Launch what is queued everywhere, then stop and join every thread.
+void stop_all()
+{
+    std::vector<Lane *> lanes;
+    {
+        std::lock_guard<std::mutex> hold(g_lock);
+        lanes.swap(g_lanes);
+        g_generation.fetch_add(1, std::memory_order_release);
+    }
+    for (Lane *l : lanes) {
+        wait_launched(l);
+        retire(l);
+    }
 }
 
 bool is_default_stream(nbh_stream_t s)
@@ -268,7 +311,13 @@ extern "C" {
 
 int nbh_launch_threads(int enable)
 {
+    if (enable < 0) {  // the process is about to end: nothing may be left to the threads
+        g_enabled.store(false, std::memory_order_release);
+        stop_all();
+        return 0;
+    }
     if (enable) {
+        register_fork_handler();
         nbh_queue_in_use.store(1, std::memory_order_release);
         g_enabled.store(true, std::memory_order_release);
     } else {

@@ -978,32 +978,50 @@ static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 namespace {
 
 constexpr int kMaxDevices = 64;
-std::atomic<void *> g_static_scratch[kMaxDevices];  // device address of `scratch`, per device
+
+// What the host knows about one device's copy of `scratch`.
+struct StaticScratch {
+    std::atomic<void *> address{nullptr};  // device address of `scratch`
+    hipEvent_t done = nullptr;             // recorded after the latest call's kernel
+    hipStream_t last = nullptr;            // the stream of that call
+    bool have_last = false;
+    bool dirty = false;                    // a call failed after its launch: the ticket may not be back at zero
+    std::mutex mu;                         // the four fields above
+};
+StaticScratch g_static[kMaxDevices];
 std::mutex g_static_mu;
 
-// Address of the current device's copy of `scratch`.
-int static_scratch(void **out)
+// The current device's entry, its array looked up and its event made on first use.
+int static_scratch(StaticScratch **out)
 {
     int dev = -1;
     NBH_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices)
         return (int)hipErrorInvalidDevice;
-    void *p = g_static_scratch[dev].load(std::memory_order_acquire);
-    if (!p) {
+    StaticScratch &st = g_static[dev];
+    if (!st.address.load(std::memory_order_acquire)) {
         std::lock_guard<std::mutex> lock(g_static_mu);
-        p = g_static_scratch[dev].load(std::memory_order_relaxed);
-        if (!p) {
+        if (!st.address.load(std::memory_order_relaxed)) {
+            void *p = nullptr;
             NBH_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
             if (!p)
                 return (int)hipErrorInvalidSymbol;
+            NBH_TRY(hipEventCreateWithFlags(&st.done, hipEventDisableTiming));
             // the array is zero when the code object is loaded, and every reduction hands
             // the ticket back at zero: nothing to clear here
-            g_static_scratch[dev].store(p, std::memory_order_release);
+            st.address.store(p, std::memory_order_release);
         }
     }
-    *out = p;
+    *out = &st;
     return 0;
 }
+
+__global__ void clear_header_kernel(unsigned *header)
+{
+    header[threadIdx.x] = 0u;
+}
+
+bool is_null_stream(hipStream_t s) { return s == nullptr || s == hipStreamLegacy; }
 
 }  // namespace
 
@@ -1012,8 +1030,41 @@ extern "C" int nbh_reduce_noalloc(int op, int dtype, const void *in, int64_t n, 
 {
     if (n > NBH_REDUCE_NOALLOC_MAX_ITEMS)
         return (int)hipErrorInvalidValue;  // stated limit of this entry point; nothing is launched
-    void *ptr = nullptr;
-    if (int rc = static_scratch(&ptr))
+    StaticScratch *st = nullptr;
+    if (int rc = static_scratch(&st))
         return rc;
-    return nbh_reduce(op, dtype, in, n, in_stride, init, out, ptr, kScratchBytes, stream);
+    void *ptr = st->address.load(std::memory_order_relaxed);
+    hipStream_t s = nbh_hip_stream(stream);
+    // Under stream capture nothing runs now: the graph's own edges order the replays, and
+    // event queries are not allowed, so the bookkeeping below is left out.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    const bool capturing = !is_null_stream(s) && s != hipStreamPerThread &&
+                           hipStreamIsCapturing(s, &capture) == hipSuccess && capture == hipStreamCaptureStatusActive;
+    if (capturing)
+        return nbh_reduce(op, dtype, in, n, in_stride, init, out, ptr, kScratchBytes, stream);
+    std::lock_guard<std::mutex> hold(st->mu);
+    // Calls on one stream run one after the other; the null stream waits for the others and
+    // they for it.  A call on ANOTHER stream while the previous call's kernel has not finished
+    // would share the ticket and the partials with it: refused instead of giving wrong results.
+    if (st->have_last && st->last != s && !is_null_stream(s) && !is_null_stream(st->last)) {
+        const hipError_t state = hipEventQuery(st->done);
+        if (state != hipSuccess)
+            return (int)state;  // hipErrorNotReady: still running
+    }
+    if (st->dirty) {  // a failed call may have left tickets drawn: start from zero again (no allocation: one launch)
+        hipLaunchKernelGGL(clear_header_kernel, dim3(1), dim3(kHeaderBytes / sizeof(unsigned)), 0, s, (unsigned *)ptr);
+        if (int rc = nbh_launch_status())
+            return rc;
+        st->dirty = false;
+    }
+    const int rc = nbh_reduce(op, dtype, in, n, in_stride, init, out, ptr, kScratchBytes, stream);
+    if (rc) {
+        st->dirty = true;
+        return rc;
+    }
+    if (hipEventRecord(st->done, s) == hipSuccess) {
+        st->last = s;
+        st->have_last = true;
+    }
+    return 0;
 }

@@ -117,8 +117,8 @@ class Driver:
         if config.DISABLE_CUDA:
             self.initialization_error = "GPU support disabled by NUMBA_DISABLE_CUDA=1"
         elif config.ENABLE_CUDASIM:
-            self.initialization_error = ("NUMBA_ENABLE_CUDASIM=1 asks for the CPU simulator, "
-                                         "which this GPU-only package does not provide")
+            self.initialization_error = ("NUMBA_ENABLE_CUDASIM=1 selects the CPU mode (numba_cuda_amd.simulator): "
+                                         "the GPU library is not loaded")
         else:
             try:
                 self.lib = _lib.load()
@@ -189,6 +189,51 @@ class Driver:
 
     def get_version(self):
         return (self.lib.nbh_version(), 0)
+
+    # --- the calling thread's active context (reference :387-407; HIP has one implicit
+    # context per device, so "pushed" contexts are a per-thread list kept here)
+    def get_active_context(self):
+        """Context manager describing what is active on the calling thread: `.devnum` and
+        `.context_handle`, both None when the thread has not selected a device yet."""
+        return _ActiveContext()
+
+    def pop_active_context(self):
+        """Take the calling thread's most recently pushed context off its stack and make the
+        one below it (if any) current; returns the popped context's handle or None."""
+        stack = _ActiveContext.pushed()
+        if not stack:
+            return None
+        popped = stack.pop()
+        if stack:
+            self.nbh_set_device(stack[-1])
+        return popped
+
+
+class _ActiveContext:
+    """What `Driver.get_active_context()` hands out (reference :420-470)."""
+
+    _tls = threading.local()
+
+    @classmethod
+    def pushed(cls):
+        try:
+            return cls._tls.stack
+        except AttributeError:
+            stack = cls._tls.stack = []
+            return stack
+
+    def __enter__(self):
+        from numba_cuda_amd.cudadrv import devices
+        stack = self.pushed()
+        self.devnum = stack[-1] if stack else devices._runtime.current_device
+        self.context_handle = self.devnum
+        return self
+
+    def __exit__(self, *exc_info):
+        return False
+
+    def __bool__(self):
+        return self.devnum is not None
 
 
 driver = Driver()
@@ -729,6 +774,19 @@ class Context:
         """Called whenever the context is fetched: lets the manager initialise (once)."""
         self._memory_manager.initialize()
         self.prepared = True
+
+    def push(self):
+        """Make this context's device current on the calling thread, remembering it on the
+        thread's stack (reference :1161-1167)."""
+        driver.nbh_set_device(self.device.id)
+        _ActiveContext.pushed().append(self.device.id)
+        self.prepare_for_use()
+
+    def pop(self):
+        """Undo the latest push; this context must be the one on top (reference :1169-1175)."""
+        stack = _ActiveContext.pushed()
+        assert stack and stack[-1] == self.device.id, "this context is not at the top of the thread's stack"
+        driver.pop_active_context()
 
     # --- memory: all of it is the memory manager's business
 

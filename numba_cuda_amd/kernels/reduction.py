@@ -125,8 +125,11 @@ def _trace(functor, answer):
     return out.name, list(log)
 
 
-def classify_functor(functor):
+def classify_functor(functor, detail=None):
     """-> "add" | "mul" | "max" | "min" | "and" | "or" | "xor", or NotImplementedError.
+    `detail`, a dict, receives "kernel_form": False when the functor is a max / min whose
+    comparison treats NaN and equal operands (signed zeros) differently from the kernels'
+    own `b if b > a else a` / `b if b < a else a`, which is what max(a, b) / min(a, b) do.
 
     The functor is run on two recording stand-ins.  `a + b` / `a * b` show up as
     one arithmetic event.  `max(a, b)` / `min(a, b)` and the equivalent
@@ -152,6 +155,9 @@ def classify_functor(functor):
                 # when "lhs <cmp_op> rhs" holds the functor returns name_t
                 greater_wins = (cmp_op in ("gt", "ge")) == (name_t == lhs)
                 verdict = "max" if greater_wins else "min"
+                # the kernels: a strict comparison that, when it holds, picks the LATER operand
+                if detail is not None:
+                    detail["kernel_form"] = cmp_op in ("gt", "lt") and name_t == "b"
     except _Unrecognised:
         verdict = None
     except Exception:
@@ -191,11 +197,15 @@ class Reduce:
         if reference_order is None:
             reference_order = bool(_config.CUDA_REDUCE_REFERENCE_ORDER)
         self._ordered = bool(reference_order)
+        self._kernel_form = True
+        self._twin = None
         try:
-            self._op = self._cache[functor]
+            self._op, self._kernel_form = self._cache[functor]
         except (KeyError, TypeError):
             try:
-                self._op = classify_functor(functor)
+                detail = {}
+                self._op = classify_functor(functor, detail)
+                self._kernel_form = detail.get("kernel_form", True)
             except NotImplementedError:
                 # not one of the operators with kernels of their own: translate it
                 try:
@@ -205,11 +215,12 @@ class Reduce:
                         "Reduce could not translate %r for the device: %s.  Translated are arithmetic, "
                         "comparisons, conditionals and math functions of the two operands." % (functor, why)) from None
             try:
-                self._cache[functor] = self._op
+                self._cache[functor] = (self._op, self._kernel_form)
             except TypeError:
                 pass
         self._custom = not isinstance(self._op, str)
-        self._native_off = self._custom or self._ordered    # cases the native passage does not take
+        # cases the native passage does not take
+        self._native_off = self._custom or self._ordered or not self._kernel_form
         self._opcode = None if self._custom else _lib.OP_CODES[self._op]
         self._codes = {}    # dtype -> (operator code, element code), filled once the pairing is checked
                             # (translated functors: dtype -> handle of the compiled operation)
@@ -273,6 +284,15 @@ class Reduce:
             return dtype.type(init)          # `res` is left untouched, as in the reference
         if self._custom:
             return self._call_translated(arr, dtype, n, res, init, stream)
+        if not self._kernel_form and dtype.kind == "f":
+            # a max / min spelled with another comparison than the kernels': the same for
+            # integers, not for NaN and signed zeros - floating point takes the translated functor
+            twin = self._twin
+            if twin is None:
+                twin = self._twin = Reduce.__new__(Reduce)
+                twin.__dict__.update(self.__dict__)
+                twin._op, twin._custom, twin._codes = _functor.trace(self._functor), True, {}
+            return twin._call_translated(arr, dtype, n, res, init, stream)
 
         codes = self._codes.get(dtype)
         if codes is None:
@@ -306,8 +326,7 @@ class Reduce:
             entry, reduce_fn = 0, lib.nbh_reduce_ordered
 
         if res is not None:
-            if res.dtype != dtype:
-                raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
+            _check_result_array(res, dtype)
             try:
                 out_ptr = res.gpu_data.device_pointer
             except AttributeError:
@@ -359,8 +378,7 @@ class Reduce:
         init_ptr = _init_buffer(dtype, init)
         lib = _driver.driver.lib
         if res is not None:
-            if res.dtype != dtype:
-                raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
+            _check_result_array(res, dtype)
             rc = lib.nbh_reduce_custom(handle, in_ptr, n, arr.strides[0], init_ptr, res.device_ctypes_pointer.value,
                                        scratch[0], scratch[1], hstream or None)
             if rc:
@@ -376,6 +394,22 @@ class Reduce:
             return cell[1][:dtype.itemsize].view(dtype)[0]
         finally:
             ctx.give_back_result_cell(cell)
+
+
+def _check_result_array(res, dtype):
+    """The reference stores the result with res[:1].copy_to_device(partials[:1])
+    (kernels/reduction.py:259-262): `res` must hold the dtype and its first slice exactly
+    one item."""
+    if res.dtype != dtype:
+        raise TypeError("res has dtype %s, expected %s" % (res.dtype, dtype))
+    if res.ndim == 0:
+        raise IndexError("too many indices for array: res is 0-dimensional")
+    head = (min(1, res.shape[0]),) + tuple(res.shape[1:])
+    items = 1
+    for extent in head:
+        items *= extent
+    if items != 1:
+        raise ValueError("incompatible shape: %s vs. (1,)" % (head,))
 
 
 # (body, element code) -> handle from nbh_reduce_compile, kept for the life of the process
@@ -418,6 +452,7 @@ def _entry_address(lib):
     try:
         if _config.CUDA_REDUCE_LAUNCH_THREADS and not lib.nbh_launch_threads(1):
             lib._launch_threads = True
+            _stop_threads_at_exit(lib)
             return ctypes.cast(lib.nbh_reduce_queued, ctypes.c_void_p).value or 0
         return ctypes.cast(lib.nbh_reduce, ctypes.c_void_p).value or 0
     except (TypeError, ctypes.ArgumentError, AttributeError):
@@ -446,10 +481,30 @@ def launch_threads(enable=True):
     if rc:
         _driver.driver.check("nbh_launch_threads", rc)
     lib._launch_threads = bool(enable)
+    if enable:
+        _stop_threads_at_exit(lib)
     try:
         lib._reduce_entry = ctypes.cast(entry, ctypes.c_void_p).value or 0
     except (TypeError, ctypes.ArgumentError):
         lib._reduce_entry = 0
+
+
+def _stop_threads_at_exit(lib):
+    """The launching threads must be idle and joined before the interpreter and the GPU runtime
+    shut down (exit hooks run in reverse order of registration: this one, registered after the
+    library was loaded, runs before the runtime's own)."""
+    if getattr(lib, "_stop_hook", False):
+        return
+    import atexit
+
+    def stop():
+        try:
+            lib.nbh_launch_threads(-1)
+        except Exception:       # noqa: BLE001 - nothing to report to at exit
+            pass
+
+    atexit.register(stop)
+    lib._stop_hook = True
 
 
 _DTYPE_CODE = {np.dtype(name): code for name, code in _lib.DTYPE_CODES.items()}

@@ -17,15 +17,14 @@ Differences in mechanism, not in results:
     comes back through a cell of device-mapped host memory.
 """
 
-import math
-
 import numpy as np
 
 from numba_cuda_amd.cudadrv import devices
 from numba_cuda_amd.cudadrv import driver as _driver
 from numba_cuda_amd import api as _api
+from numba_cuda_amd import _xoroshiro_host as _host
 
-xoroshiro128p_dtype = np.dtype([("s0", np.uint64), ("s1", np.uint64)], align=True)
+xoroshiro128p_dtype = _host.xoroshiro128p_dtype
 
 UNIFORM = 1
 NORMAL = 2
@@ -157,90 +156,60 @@ def init_xoroshiro128p_state(states, index, seed):
         devices.get_context()
         _driver.driver.nbh_xoro_init_states(_record_address(states, index), 1, int(seed) & _M64, 0, None)
         return
-    z = (int(seed) + 0x9E3779B97F4A7C15) & _M64
-    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
-    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
-    z ^= z >> 31
-    states[int(index)]["s0"] = z
-    states[int(index)]["s1"] = z
+    _host.init_state(states, index, seed)
 
 
-def rotl(x, k):
-    x = int(x) & _M64
-    return ((x << k) & _M64) | (x >> (64 - k))
+rotl = _host.rotl
+uint64_to_unit_float64 = _host.uint64_to_unit_float64
+uint64_to_unit_float32 = _host.uint64_to_unit_float32
+TWO_PI_FLOAT32 = _host.TWO_PI_FLOAT32
+TWO_PI_FLOAT64 = _host.TWO_PI_FLOAT64
 
 
 def xoroshiro128p_next(states, index):
     """Next uint64 of generator `index`; advances it."""
     if _driver.is_device_memory(states):
         return _on_device(states, index, _ONE_NEXT)
-    index = int(index)
-    s0 = int(states[index]["s0"])
-    s1 = int(states[index]["s1"])
-    result = (s0 + s1) & _M64
-    s1 ^= s0
-    states[index]["s0"] = rotl(s0, 55) ^ s1 ^ ((s1 << 14) & _M64)
-    states[index]["s1"] = rotl(s1, 36)
-    return np.uint64(result)
+    return _host.next_u64(states, index)
 
 
 def xoroshiro128p_jump(states, index):
     """Advance generator `index` by 2**64 steps."""
     if _driver.is_device_memory(states):
         return _on_device(states, index, _ONE_JUMP)
-    index = int(index)
-    s0 = s1 = 0
-    for word in (0xBEAC0467EBA5FACB, 0xD86B048B86AA9922):
-        for b in range(64):
-            if (word >> b) & 1:
-                s0 ^= int(states[index]["s0"])
-                s1 ^= int(states[index]["s1"])
-            xoroshiro128p_next(states, index)
-    states[index]["s0"] = s0
-    states[index]["s1"] = s1
-
-
-def uint64_to_unit_float64(x):
-    return np.float64((int(x) >> 11) * (1.0 / (1 << 53)))
-
-
-def uint64_to_unit_float32(x):
-    return np.float32(uint64_to_unit_float64(x))
+    _host.jump(states, index)
 
 
 def xoroshiro128p_uniform_float32(states, index):
     if _driver.is_device_memory(states):
         return _on_device(states, index, _ONE_UNIFORM_F32)
-    return uint64_to_unit_float32(xoroshiro128p_next(states, index))
+    return _host.uniform_float32(states, index)
 
 
 def xoroshiro128p_uniform_float64(states, index):
     if _driver.is_device_memory(states):
         return _on_device(states, index, _ONE_UNIFORM_F64)
-    return uint64_to_unit_float64(xoroshiro128p_next(states, index))
-
-
-TWO_PI_FLOAT32 = np.float32(2 * math.pi)
-TWO_PI_FLOAT64 = np.float64(2 * math.pi)
+    return _host.uniform_float64(states, index)
 
 
 def xoroshiro128p_normal_float32(states, index):
     """Box-Muller (cosine branch) in float32; uses two draws."""
     if _driver.is_device_memory(states):
         return _on_device(states, index, _ONE_NORMAL_F32)
-    u1 = xoroshiro128p_uniform_float32(states, index)
-    u2 = xoroshiro128p_uniform_float32(states, index)
-    with np.errstate(divide="ignore"):
-        r = np.sqrt(-np.float32(2.0) * np.log(u1))
-    return np.float32(r * np.cos(TWO_PI_FLOAT32 * u2))
+    return _host.normal_float32(states, index)
 
 
 def xoroshiro128p_normal_float64(states, index):
     """Box-Muller (cosine branch); float32 uniforms and logarithm, float64 rest."""
     if _driver.is_device_memory(states):
         return _on_device(states, index, _ONE_NORMAL_F64)
-    u1 = xoroshiro128p_uniform_float32(states, index)
-    u2 = xoroshiro128p_uniform_float32(states, index)
-    with np.errstate(divide="ignore"):
-        r = np.sqrt(-np.float64(2.0) * np.float64(np.log(u1)))
-    return np.float64(r * np.cos(TWO_PI_FLOAT64 * np.float64(u2)))
+    return _host.normal_float64(states, index)
+
+
+def init_xoroshiro128p_states_cpu(states, seed, subsequence_start):
+    """Fill a HOST array of states exactly as init_xoroshiro128p_states fills a device
+    array (the reference's helper of this name, random.py:241-257, builds them as a
+    sequential chain; here the chain is unrolled by doubling with GF(2) jump matrices)."""
+    if states.ndim != 1 or states.dtype.itemsize != 16:
+        raise TypeError("states must be a 1D array of xoroshiro128p_dtype")
+    _host.init_states_cpu(states, seed, subsequence_start)

@@ -51,8 +51,8 @@ def fake_gpu(monkeypatch):
     d.lib, d.is_initialized, d.initialization_error, d.pid = lib, True, None, os.getpid()
     d._devices = {}                               # a table of its own for the fake devices
     devices._runtime._tls.__dict__.clear()
-    if "lst" in devices.gpus.__dict__:
-        del devices.gpus.__dict__["lst"]
+    devices.gpus._entries = None                  # the device list is asked for again, from the fake library
+    drv._ActiveContext._tls.__dict__.clear()
     monkeypatch.setattr(drv, "_memory_manager", None)
     try:
         yield lib
@@ -64,5 +64,5 @@ def fake_gpu(monkeypatch):
         for name in [k for k in d.__dict__ if k.startswith("nbh_")]:
             del d.__dict__[name]
         devices._runtime._tls.__dict__.clear()
-        if "lst" in devices.gpus.__dict__:
-            del devices.gpus.__dict__["lst"]
+        devices.gpus._entries = None
+        drv._ActiveContext._tls.__dict__.clear()

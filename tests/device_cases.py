@@ -73,4 +73,46 @@ def gpus_list_and_memory_info(cuda):
     assert np.allclose(a, back)
 
 
-ALL = [select_device_in_fresh_threads, select_and_close_repeatedly, gpus_list_and_memory_info]
+def active_context_and_push_pop(cuda):
+    # test_context_stack.py:48-68 (the active context of a fresh thread is empty; after a device is
+    # selected it names that device) and cudadrv/driver.py:1161-1175 (push / pop in LIFO order)
+    seen = {}
+
+    def fresh_thread():
+        with driver.driver.get_active_context() as ac:
+            seen["devnum"], seen["truth"] = ac.devnum, bool(ac)
+
+    _in_threads(fresh_thread, 1)
+    assert seen == {"devnum": None, "truth": False}
+    cuda.select_device(0)
+    with driver.driver.get_active_context() as ac:
+        assert ac.devnum == 0 and ac.context_handle is not None and ac
+    ctx = cuda.current_context()
+    assert driver.driver.pop_active_context() is None       # nothing was pushed on this thread
+    ctx.push()
+    ctx.push()
+    with driver.driver.get_active_context() as ac:
+        assert ac.devnum == 0
+    ctx.pop()
+    ctx.pop()
+    try:
+        ctx.pop()
+    except AssertionError:
+        pass
+    else:
+        raise AssertionError("pop of a context that is not on the stack must fail")
+    d = cuda.to_device(np.arange(4))
+    assert d.copy_to_host().tolist() == [0, 1, 2, 3]
+
+
+def auto_device_helper(cuda):
+    # api.py:522-523
+    host = np.arange(5.0)
+    dev, fresh = cuda._auto_device(host)
+    assert fresh and dev.copy_to_host().tolist() == host.tolist()
+    again, fresh = cuda._auto_device(dev)
+    assert again is dev and not fresh
+
+
+ALL = [select_device_in_fresh_threads, select_and_close_repeatedly, gpus_list_and_memory_info,
+       active_context_and_push_pop, auto_device_helper]

@@ -9,11 +9,14 @@
 #include <atomic>
 #include <chrono>
 #include <cstdio>
+#include <csignal>
 #include <cstdlib>
 #include <map>
 #include <mutex>
 #include <thread>
 #include <vector>
+#include <sys/wait.h>
+#include <unistd.h>
 extern "C" int nbh_launch_threads(int enable);
 extern "C" int nbh_launch_threads_wait(nbh_stream_t stream);
 extern "C" int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
@@ -21,10 +24,12 @@ extern "C" int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, i
 static std::mutex g_m;
 static std::map<void *, std::vector<int64_t>> g_seen;   // per stream: the n of each launch, in order
 static std::atomic<long> g_calls{0};
+static std::atomic<bool> g_block{false};   // holds the launching threads inside a launch
 extern "C" int nbh_reduce(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                           void *scratch, size_t scratch_bytes, nbh_stream_t stream)
 {
     (void)nbh_hip_stream(stream);   // what the real one does first
+    while (g_block.load()) std::this_thread::sleep_for(std::chrono::milliseconds(1));
     if (in_stride == 6) return 1;
     {
         std::lock_guard<std::mutex> h(g_m);
@@ -79,7 +84,40 @@ int main()
     nbh_reduce_queued(0, 2, &dummy_in, 3, 6, &init, &o, &scratch, 4, streams[0]);
     nbh_queue_drain(streams[0]);
     if (nbh_queue_take_status(streams[0]) != 1 || nbh_queue_take_status(streams[0]) != 0) { printf("status\n"); return 1; }
+    // A fork while launches are queued: the child has no launching threads; every call that waits
+    // for queues must return there, and launches go straight through (feature off in the child).
+    g_block.store(true);
+    for (int i = 0; i < 50; ++i) nbh_reduce_queued(0, 2, &dummy_in, 9, 4, &init, &o, &scratch, 4, streams[1]);
+    const pid_t child = fork();
+    if (child == 0) {
+        g_block.store(false);
+        nbh_queue_drain(nullptr);
+        nbh_queue_drain(streams[1]);
+        nbh_launch_threads_wait(streams[1]);
+        int64_t mine = 0;
+        if (nbh_reduce_queued(0, 2, &dummy_in, 11, 4, &init, &mine, &scratch, 4, streams[1]) || mine != 11) _exit(3);
+        nbh_queue_forget(streams[1]);
+        nbh_launch_threads(-1);
+        _exit(0);
+    }
+    int status = -1;
+    for (int waited = 0; waited < 200; ++waited) {          // 20 s at most: a hang in the child is the failure
+        if (waitpid(child, &status, WNOHANG) == child) break;
+        std::this_thread::sleep_for(std::chrono::milliseconds(100));
+        status = -1;
+    }
+    g_block.store(false);
+    if (status == -1) { kill(child, SIGKILL); printf("child hung after fork\n"); return 1; }
+    if (!WIFEXITED(status) || WEXITSTATUS(status) != 0) { printf("child failed: %d\n", status); return 1; }
+    nbh_queue_drain(nullptr);
     for (void *st : streams) nbh_queue_forget(st);
+    // explicit stop at the end of a process: queued work is launched, the threads are joined, and
+    // the switch can be used again afterwards
+    nbh_launch_threads(1);
+    for (int i = 0; i < 100; ++i) nbh_reduce_queued(0, 2, &dummy_in, 4, 4, &init, &o, &scratch, 4, streams[2]);
+    const long before = g_calls.load();
+    nbh_launch_threads(-1);
+    if (g_calls.load() < before || o != 4) { printf("stop lost launches\n"); return 1; }
     printf("ok, %ld launches\n", g_calls.load());
     return 0;
 }

@@ -525,3 +525,58 @@ def test_per_thread_default_stream_keeps_scratch_per_thread():
     for t in threads:
         t.join()
     assert not wrong, wrong
+
+
+def test_by_the_book_publication_build_gives_the_same_bits():
+    """libnbhip_release_publish.so is the same library with the reduction kernels publishing
+    their partials through ordinary stores and a release at agent scope
+    (-DNBH_REDUCE_RELEASE_PUBLISH=1) instead of the written-through atomic stores the shipped
+    build relies on.  Loaded beside the shipped library and driven through the C ABI on the same
+    device memory: integer sums from 1200 back-to-back launches of changing sizes must equal the
+    exact prefix-sum differences and the shipped build's results, bit for bit."""
+    import ctypes
+    import os
+    from numba_cuda_amd import _build, _lib
+    from numba_cuda_amd.cudadrv import driver as drv
+    if not os.path.exists(_build.RELEASE_PUBLISH_LIB):
+        pytest.fail("%s is missing: __graft_entry__.build() makes it" % _build.RELEASE_PUBLISH_LIB)
+    other = ctypes.CDLL(_build.RELEASE_PUBLISH_LIB)
+    for name in ("nbh_reduce", "nbh_reduce_scratch_bytes", "nbh_stream_synchronize"):
+        getattr(other, name).restype, getattr(other, name).argtypes = _lib.SIGNATURES[name]
+    cuda.current_context()
+    shipped = drv.driver.lib
+    rng = np.random.default_rng(123)
+    calls, n_max = 1200, 6_000_000
+    base = rng.integers(-2**40, 2**40, n_max + 4096, dtype=np.int64)
+    d = cuda.to_device(base)
+    offs = rng.integers(0, 4096, calls)
+    sizes = rng.integers(3000, n_max, calls)
+    out_a, out_b = cuda.device_array(calls, np.int64), cuda.device_array(calls, np.int64)
+    nbytes = other.nbh_reduce_scratch_bytes()
+    assert nbytes == shipped.nbh_reduce_scratch_bytes()
+    scratch_a = cuda.to_device(np.zeros(nbytes, np.uint8))
+    scratch_b = cuda.to_device(np.zeros(nbytes, np.uint8))
+    stream = cuda.stream()
+    code, op = _lib.DTYPE_CODES["int64"], _lib.OP_CODES["add"]
+    inits = np.arange(calls, dtype=np.int64)
+    for i in range(calls):
+        src = d.device_ctypes_pointer.value + 8 * int(offs[i])
+        for lib, out, scratch in ((shipped, out_a, scratch_a), (other, out_b, scratch_b)):
+            rc = lib.nbh_reduce(op, code, src, int(sizes[i]), 8, inits[i:i + 1].ctypes.data,
+                                out.device_ctypes_pointer.value + 8 * i, scratch.device_ctypes_pointer.value, nbytes,
+                                stream.handle)
+            assert rc == 0
+    stream.synchronize()
+    csum = np.concatenate([[0], np.cumsum(base)])
+    want = csum[offs + sizes] - csum[offs] + np.arange(calls)
+    got_a, got_b = out_a.copy_to_host(), out_b.copy_to_host()
+    assert (got_b == want).all() and (got_a == got_b).all()
+    # floating point: the same kernels and grid, so the same bits
+    f = cuda.to_device(rng.standard_normal(3_000_001).astype(np.float32))
+    fa, fb = cuda.device_array(1, np.float32), cuda.device_array(1, np.float32)
+    zero = np.zeros(1, np.float32)
+    for lib, out, scratch in ((shipped, fa, scratch_a), (other, fb, scratch_b)):
+        assert lib.nbh_reduce(op, _lib.DTYPE_CODES["float32"], f.device_ctypes_pointer.value, f.size, 4, zero.ctypes.data,
+                              out.device_ctypes_pointer.value, scratch.device_ctypes_pointer.value, nbytes, stream.handle) == 0
+    stream.synchronize()
+    assert fa.copy_to_host().tobytes() == fb.copy_to_host().tobytes()

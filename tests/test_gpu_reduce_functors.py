@@ -237,3 +237,32 @@ def test_untranslatable_functor_is_refused_when_the_object_is_made():
         cuda.Reduce(FC.BY_NAME["xor_and_flip"].functor)(np.zeros(4, np.float32))
     with pytest.raises(NotImplementedError, match="dtype"):
         cuda.Reduce(FC.BY_NAME["sum_plus_one"].functor)(np.zeros(4, np.complex64))
+
+
+def test_max_min_spelled_with_other_comparisons_keep_their_own_nan_rule():
+    """`a if a >= b else b` and its relatives are max / min for integers (native kernels) but drop
+    or keep NaN differently from `max(a, b)`: on floating point they run as translated functors,
+    whose comparison is the functor's own.  With NaN among the operands these functors are not
+    associative, so only inputs of one or two items have an answer that does not depend on the
+    order of association: those are compared with the functor applied as the reference applies
+    it (oracle.cref.functor_tree), NaN for NaN; NaN-free inputs of every size bit for bit."""
+    spellings = [lambda a, b: a if a >= b else b, lambda a, b: a if a > b else b,
+                 lambda a, b: b if b >= a else a, lambda a, b: a if a < b else b, lambda a, b: a if a <= b else b]
+    rng = np.random.default_rng(77)
+    nan = np.float32(np.nan)
+    for k, functor in enumerate(spellings):
+        red = cuda.Reduce(functor)
+        assert not red._kernel_form
+        for data in ([nan], [1.0], [nan, 2.0], [2.0, nan], [nan, nan], [0.0, -0.0], [-0.0, 0.0]):
+            for init in (0.25, nan, -0.0):
+                data32 = np.array(data, np.float32)
+                _say("spelling", k, data, init)
+                want = cref.functor_tree(functor, data32, init)
+                got = red(data32, init=init)
+                assert got.tobytes() == want.tobytes() or (np.isnan(got) and np.isnan(want)), (k, data, init, got, want)
+        for n in (65, 1000, 70001):
+            clean = rng.standard_normal(n).astype(np.float32)
+            assert red(clean, init=0.25).tobytes() == cref.functor_tree(functor, clean, 0.25).tobytes()
+        # integers: the native kernels, exact
+        ints = rng.integers(-1000, 1000, 5000).astype(np.int32)
+        assert red(ints, init=0) == cref.functor_tree(functor, ints, 0)

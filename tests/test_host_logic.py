@@ -115,7 +115,30 @@ def test_reduce_object_caches_its_operator():
     f = lambda a, b: a + b      # noqa: E731
     r1, r2 = cuda.Reduce(f), cuda.reduce(f)
     assert r1._op == r2._op == "add"
-    assert cuda.Reduce._cache[f] == "add"
+    assert cuda.Reduce._cache[f] == ("add", True)
+
+
+@pytest.mark.parametrize("functor,kernel_form", [
+    (lambda a, b: max(a, b), True), (max, True), (lambda a, b: b if b > a else a, True),
+    (lambda a, b: b if a < b else a, True), (lambda a, b: min(a, b), True), (lambda a, b: b if b < a else a, True),
+    (lambda a, b: b if a > b else a, True),
+    # the same operators for integers; NaN or equal operands come out differently
+    (lambda a, b: a if a > b else b, False), (lambda a, b: a if a >= b else b, False),
+    (lambda a, b: b if b >= a else a, False), (lambda a, b: a if a < b else b, False),
+    (lambda a, b: b if a >= b else a, False),
+])
+def test_comparison_spellings_that_differ_from_the_kernels_are_told_apart(functor, kernel_form):
+    detail = {}
+    assert classify_functor(functor, detail) in ("max", "min")
+    assert detail.get("kernel_form", True) is kernel_form
+    r = cuda.Reduce(functor)
+    assert r._kernel_form is kernel_form and r._native_off is (not kernel_form)
+    # what Python itself makes of NaN with this functor, against the kernels' rule
+    nan = float("nan")
+    op = classify_functor(functor)
+    kernel = (lambda a, b: b if b > a else a) if op == "max" else (lambda a, b: b if b < a else a)
+    same = all(repr(functor(a, b)) == repr(kernel(a, b)) for a, b in ((nan, 1.0), (1.0, nan), (0.0, -0.0), (-0.0, 0.0)))
+    assert same is kernel_form
 
 
 # ---------------------------------------------------------------- argument normalisation

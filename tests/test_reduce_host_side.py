@@ -150,6 +150,27 @@ def test_res_argument_bypasses_the_cells_and_returns_none(fake_gpu):
     assert res.copy_to_host()[0] == 15
 
 
+def test_res_must_hold_one_item_in_its_first_slice(fake_gpu):
+    """The reference writes the result with res[:1].copy_to_device(partials[:1])
+    (kernels/reduction.py:259-262): an empty or wider `res` is an error there, not a write past its end."""
+    record = _install_recording_reduce(fake_gpu)
+    add = cuda.Reduce(lambda a, b: a + b)
+    d = cuda.to_device(np.arange(10, dtype=np.int64))
+    with pytest.raises(ValueError, match="incompatible shape"):
+        add(d, res=cuda.device_array(0, np.int64))
+    with pytest.raises(ValueError, match="incompatible shape"):
+        add(d, res=cuda.device_array((2, 3), np.int64))
+    with pytest.raises(IndexError):
+        add(d, res=cuda.device_array((), np.int64))
+    with pytest.raises(TypeError, match="dtype"):
+        add(d, res=cuda.device_array(1, np.int32))
+    assert record == []
+    column = cuda.device_array((4, 1), np.int64)         # its first slice is one item: accepted
+    add(d, res=column)
+    fake_gpu.nbh_stream_synchronize(None)
+    assert column.copy_to_host()[0, 0] == 45 and len(record) == 1
+
+
 def test_init_values_are_told_apart_by_their_bits():
     f64 = np.dtype(np.float64)
     plus = reduction._init_buffer(f64, 0.0)

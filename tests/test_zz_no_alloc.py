@@ -114,3 +114,61 @@ def test_noalloc_rejects_sizes_beyond_its_limit_and_bad_arguments():
     assert lib.nbh_reduce_noalloc(0, f32, p, 4, 4, init.ctypes.data, o, None) == 0
     cuda.synchronize()
     assert out.copy_to_host()[0] == 4.0
+
+
+def test_calls_allocate_nothing():
+    """Free device memory (and, with the pooling manager, what the pool holds) is the same
+    after a loop of calls as after the first one: no hipMalloc behind this entry point."""
+    import ctypes
+    cuda.current_context()
+    lib = drv.driver.lib
+    a = np.random.default_rng(3).integers(-1000, 1000, 1 << 20, dtype=np.int64)
+    d = cuda.to_device(a)
+    out = cuda.device_array(1, np.int64)
+    init = np.zeros(1, np.int64)
+    code, op = _lib.DTYPE_CODES["int64"], _lib.OP_CODES["add"]
+
+    def call(n):
+        assert lib.nbh_reduce_noalloc(op, code, d.device_ctypes_pointer.value, n, 8, init.ctypes.data,
+                                      out.device_ctypes_pointer.value, None) == 0
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert lib.nbh_mem_info(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    call(a.size)                      # first call on the device: looks the array up
+    cuda.synchronize()
+    before = free_bytes()
+    for i in range(200):
+        call(a.size - 17 * i)
+    cuda.synchronize()
+    assert free_bytes() == before
+    assert out.copy_to_host()[0] == a[:a.size - 17 * 199].sum()
+
+
+def test_overlap_on_another_stream_is_refused_not_raced():
+    """A call on a second stream while the first stream's call is still running would share the
+    ticket: hipErrorNotReady instead; after the first stream is done the same call goes through."""
+    cuda.current_context()
+    lib = drv.driver.lib
+    big = cuda.to_device(np.ones(1 << 28, dtype=np.int32))
+    small = cuda.to_device(np.arange(1000, dtype=np.int32))
+    out_big, out_small = cuda.device_array(1, np.int32), cuda.device_array(1, np.int32)
+    init = np.zeros(1, np.int32)
+    code, op = _lib.DTYPE_CODES["int32"], _lib.OP_CODES["add"]
+    s1, s2 = cuda.stream(), cuda.stream()
+    cuda.synchronize()
+    for _ in range(3):                # about half a millisecond of work on the first stream
+        assert lib.nbh_reduce_noalloc(op, code, big.device_ctypes_pointer.value, big.size, 4, init.ctypes.data,
+                                      out_big.device_ctypes_pointer.value, s1.handle) == 0
+    rc = lib.nbh_reduce_noalloc(op, code, small.device_ctypes_pointer.value, small.size, 4, init.ctypes.data,
+                                out_small.device_ctypes_pointer.value, s2.handle)
+    HIP_ERROR_NOT_READY = 600
+    assert rc == HIP_ERROR_NOT_READY
+    s1.synchronize()
+    assert out_big.copy_to_host()[0] == 1 << 28
+    assert lib.nbh_reduce_noalloc(op, code, small.device_ctypes_pointer.value, small.size, 4, init.ctypes.data,
+                                  out_small.device_ctypes_pointer.value, s2.handle) == 0
+    s2.synchronize()
+    assert out_small.copy_to_host()[0] == 499500
