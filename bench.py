@@ -269,9 +269,9 @@ def _workload(name, cuda):
         def extras():
             """Where a call's time goes: the issuing loop alone (no waiting), the same
             4096 launches of this kernel issued through the bare native call with precomputed
-            integer arguments - what the runtime's launch path costs per call, the floor
-            under any per-call interface on one host thread - and the whole step again with
-            the launches handed to a launching thread per stream."""
+            integer arguments on the calling thread - what the runtime's launch path costs per
+            call, the floor under any per-call interface on one host thread - and the whole step
+            again with the launching threads switched off (every launch made by the caller)."""
             from numba_cuda_amd.cudadrv import driver as drv
             from numba_cuda_amd.kernels import reduction
             cuda.synchronize()
@@ -280,35 +280,34 @@ def _workload(name, cuda):
                 add(views[r], res=slots[r], stream=streams[r & 3])
             issue = time.perf_counter() - t0
             cuda.synchronize()
-            lib, ctx = drv.driver.lib, cuda.current_context()
-            entry = lib._reduce_entry
-            scratch = [ctx.reduce_scratch(s.handle) for s in streams]
-            handles = [s.handle for s in streams]
-            init_ptr = reduction._init_buffer(np.dtype(np.float32), 0)
-            a, o = dm.gpu_data.device_pointer, out.gpu_data.device_pointer
-            args = [(entry, 0, 8, a + r * cols * 4, cols, 4, init_ptr, o + 4 * r, scratch[r & 3][0], scratch[r & 3][1],
-                     handles[r & 3]) for r in range(rows)]
-            call = drv._hostbuf.call_reduce
-            t0 = time.perf_counter()
-            for t in args:
-                call(*t)
-            floor = time.perf_counter() - t0
-            cuda.synchronize()
-            # the same step with a launching thread per stream (opt-in mode, off otherwise)
-            reduction.launch_threads(True)
+            reduction.launch_threads(False)
             try:
+                lib, ctx = drv.driver.lib, cuda.current_context()
+                entry = lib._reduce_entry
+                handles = [s._h for s in streams]      # `_h`: the streams stay inside the package
+                scratch = [ctx.reduce_scratch(h) for h in handles]
+                init_ptr = reduction._init_buffer(np.dtype(np.float32), 0)
+                a, o = dm.gpu_data.device_pointer, out.gpu_data.device_pointer
+                args = [(entry, 0, 8, a + r * cols * 4, cols, 4, init_ptr, o + 4 * r, scratch[r & 3][0], scratch[r & 3][1],
+                         handles[r & 3]) for r in range(rows)]
+                call = drv._hostbuf.call_reduce
+                t0 = time.perf_counter()
+                for t in args:
+                    call(*t)
+                floor = time.perf_counter() - t0
+                cuda.synchronize()
                 step(0)
                 cuda.synchronize()
                 t0 = time.perf_counter()
                 for k in range(3):
                     step(k)
                 cuda.synchronize()
-                queued = (time.perf_counter() - t0) / (3 * rows)
+                direct = (time.perf_counter() - t0) / (3 * rows)
             finally:
-                reduction.launch_threads(False)
+                reduction.launch_threads(True)
             return {"issue_us_per_call": round(issue / rows * 1e6, 3),
                     "native_launch_us_per_call": round(floor / rows * 1e6, 3),
-                    "launch_threads_us_per_call": round(queued * 1e6, 3)}
+                    "caller_thread_launches_us_per_call": round(direct * 1e6, 3)}
 
         return dict(desc="4096 x (65536 fp32) row sums round-robin over 4 streams, seed 3", dtype="f32",
                     algo_bytes=host.nbytes, units=rows, step=step, stream=streams[0], host=host,

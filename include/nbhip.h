@@ -204,9 +204,13 @@ int nbh_reduce_ordered(int op, int dtype, const void *in, int64_t n, int64_t in_
  *     does the same and then joins every thread: for the end of a process, before the GPU
  *     runtime's own exit handlers run.  A forked child starts with the mode off and no queues.
  *   - nbh_launch_threads_wait(stream) waits until what has been queued for `stream` (0: for
- *     every stream) is in its stream, without waiting for the device. */
+ *     every stream) is in its stream, without waiting for the device.
+ *   - nbh_stream_pin_direct(stream): the stream's handle is about to be used by code outside
+ *     the library.  What is queued for it is launched, and from then on its reductions are
+ *     launched on the calling thread whatever the mode (until the stream is destroyed). */
 int nbh_launch_threads(int enable);
 int nbh_launch_threads_wait(nbh_stream_t stream);
+int nbh_stream_pin_direct(nbh_stream_t stream);
 int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                       void *scratch, size_t scratch_bytes, nbh_stream_t stream);
 

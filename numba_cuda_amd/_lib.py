@@ -70,6 +70,7 @@ SIGNATURES = {
     "nbh_reduce_queued": (c_int, [c_int, c_int, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_size, c_vp]),
     "nbh_launch_threads": (c_int, [c_int]),
     "nbh_launch_threads_wait": (c_int, [c_vp]),
+    "nbh_stream_pin_direct": (c_int, [c_vp]),
     "nbh_reduce_noalloc": (c_int, [c_int, c_int, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp]),
     "nbh_reduce_compile": (c_int, [c_int, ctypes.c_char_p, ctypes.POINTER(c_vp), ctypes.c_char_p, c_size]),
     "nbh_reduce_op_dtype": (c_int, [c_vp]),

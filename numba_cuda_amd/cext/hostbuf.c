@@ -351,7 +351,7 @@ PyMODINIT_FUNC PyInit__hostbuf(void)
     if (!m)
         return NULL;
     str_rk = PyUnicode_InternFromString("_rk");
-    str_handle = PyUnicode_InternFromString("handle");
+    str_handle = PyUnicode_InternFromString("_h");
     str_ctx = PyUnicode_InternFromString("ctx");
     str_prepared = PyUnicode_InternFromString("prepared");
     str_scratch = PyUnicode_InternFromString("_scratch");

@@ -38,9 +38,10 @@ def reload_config():
     # not in the reference: 1 makes Reduce apply its operator in the association order of the
     # reference's kernels, so that floating-point results have the reference's bits
     g["CUDA_REDUCE_REFERENCE_ORDER"] = _readenv("NUMBA_CUDA_REDUCE_REFERENCE_ORDER", int, 0)
-    # not in the reference: 1 hands the kernel launches of Reduce(...)(arr, res=..., stream=s) to a
-    # launching thread per stream (kernels/reduction.py launch_threads)
-    g["CUDA_REDUCE_LAUNCH_THREADS"] = _readenv("NUMBA_CUDA_REDUCE_LAUNCH_THREADS", int, 0)
+    # not in the reference: 1 (the default) hands the kernel launches of Reduce(...)(arr, res=..., stream=s)
+    # on streams made by cuda.stream() to a launching thread per stream, until the stream's handle is
+    # read by code outside the package (kernels/reduction.py launch_threads); 0 launches on the caller's thread
+    g["CUDA_REDUCE_LAUNCH_THREADS"] = _readenv("NUMBA_CUDA_REDUCE_LAUNCH_THREADS", int, 1)
 
 
 reload_config()

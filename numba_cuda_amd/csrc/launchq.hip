@@ -55,10 +55,12 @@ struct Lane {
     nbh_stream_t stream = nullptr;
     int device = 0;
     pid_t owner = 0;              // the process that started the thread (a forked child has none)
+    bool has_thread = false;      // set once, before the lane is published
     Job ring[kRing];
     std::atomic<uint64_t> pushed{0}, issued{0};
     std::atomic<int> status{0};   // first failure since the last report
     std::atomic<bool> stop{false}, asleep{false};
+    std::atomic<bool> direct{false};  // the stream's handle has left the library: launches go straight to the runtime
     std::mutex push_lock;         // several host threads may use one stream
     std::mutex sleep_lock;
     std::condition_variable wake;
@@ -131,7 +133,7 @@ void rouse(Lane *lane)
 }
 
 // The lane of a stream, from a small per-thread cache; made (with its thread) on first use.
-Lane *lane_of(nbh_stream_t stream, bool make)
+Lane *lane_of(nbh_stream_t stream, bool make, bool with_thread = true)
 {
     struct Cached {
         nbh_stream_t stream;
@@ -162,7 +164,11 @@ Lane *lane_of(nbh_stream_t stream, bool make)
             found->owner = getpid();
             if (hipGetDevice(&found->device) != hipSuccess)
                 found->device = 0;
-            found->worker = std::thread(run, found);
+            found->has_thread = with_thread;
+            if (with_thread)
+                found->worker = std::thread(run, found);
+            else
+                found->direct.store(true);
             g_lanes.push_back(found);
             g_generation.fetch_add(1, std::memory_order_release);  // other threads may have cached "no lane"
         }
@@ -176,8 +182,8 @@ Lane *lane_of(nbh_stream_t stream, bool make)
 
 void wait_launched(Lane *lane)
 {
-    if (lane->owner != getpid())
-        return;  // a forked child: the thread that would launch them does not exist here
+    if (lane->owner != getpid() || !lane->has_thread)
+        return;  // a forked child, or a lane that never had a thread: nothing is queued
     const uint64_t upto = lane->pushed.load(std::memory_order_acquire);
     if (lane->issued.load(std::memory_order_acquire) >= upto)
         return;
@@ -189,7 +195,8 @@ void wait_launched(Lane *lane)
 void retire(Lane *lane)
 {
     if (lane->owner != getpid()) {  // a forked child: the thread does not exist here
-        lane->worker.detach();
+        if (lane->worker.joinable())
+            lane->worker.detach();
         return;                     // the lane is left behind
     }
     lane->stop.store(true, std::memory_order_release);
@@ -330,6 +337,28 @@ int nbh_launch_threads(int enable)
     return 0;
 }
 
+// The stream's handle is about to be used by code outside the library, which cannot know
+// about the queue: launch what is queued, and from now on launch on the calling thread.
+int nbh_stream_pin_direct(nbh_stream_t stream)
+{
+    if (is_default_stream(stream))
+        return 0;
+    if (!nbh_queue_in_use.load(std::memory_order_acquire) && !g_enabled.load(std::memory_order_acquire)) {
+        // nothing has ever been queued; remember the stream all the same, the mode may be switched on later
+        register_fork_handler();
+        nbh_queue_in_use.store(1, std::memory_order_release);
+    }
+    Lane *lane = lane_of(stream, true, false);
+    if (!lane)
+        return 0;
+    {
+        std::lock_guard<std::mutex> hold(lane->push_lock);
+        lane->direct.store(true, std::memory_order_relaxed);
+    }
+    wait_launched(lane);
+    return 0;
+}
+
 int nbh_launch_threads_wait(nbh_stream_t stream)
 {
     if (nbh_queue_in_use.load(std::memory_order_relaxed))
@@ -346,7 +375,11 @@ int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, int64_t in_s
     Lane *lane = lane_of(stream, true);
     if (!lane)
         return nbh_reduce(op, dtype, in, n, in_stride, init, out, scratch, scratch_bytes, stream);
-    std::lock_guard<std::mutex> hold(lane->push_lock);
+    std::unique_lock<std::mutex> hold(lane->push_lock);
+    if (lane->direct.load(std::memory_order_relaxed)) {
+        hold.unlock();
+        return nbh_reduce(op, dtype, in, n, in_stride, init, out, scratch, scratch_bytes, stream);
+    }
     const uint64_t at = lane->pushed.load(std::memory_order_relaxed);
     if (at - lane->issued.load(std::memory_order_acquire) >= kRing) {
         rouse(lane);

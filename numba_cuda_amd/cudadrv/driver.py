@@ -689,6 +689,7 @@ def _ensure_memory_manager():
 # Context
 # --------------------------------------------------------------------------------
 
+HIP_STREAM_LEGACY = 1
 HIP_STREAM_PER_THREAD = 2
 
 
@@ -1304,44 +1305,65 @@ class _SyncOnExit:
 
 
 class Stream:
-    """A HIP stream; handle 0 is the legacy default stream (reference :1890-2017)."""
+    """A HIP stream; handle 0 is the legacy default stream (reference :1890-2017).
+
+    The package keeps the raw handle in `_h`.  Whoever reads `handle`, converts the stream to
+    an int or asks for `__cuda_stream__` is about to use the stream outside the package, where
+    the launching threads' queues (kernels/reduction.py) are unknown: the stream's queue is
+    launched first and its reductions are launched directly from then on."""
 
     def __init__(self, handle, finalizer=None, external=False):
-        self.handle = int(handle or 0)
+        self._h = int(handle or 0)
         self.external = external
+        self._exported = self._h in (0, HIP_STREAM_LEGACY, HIP_STREAM_PER_THREAD)   # default streams are never queued
+        if external:
+            self._export()
         if finalizer is not None:
             weakref.finalize(self, finalizer)
+
+    def _export(self):
+        self._exported = True
+        if driver.is_initialized and driver.lib is not None:
+            pin = getattr(driver.lib, "nbh_stream_pin_direct", None)
+            if pin is not None:
+                pin(self._h or None)
+
+    @property
+    def handle(self):
+        if not self._exported:
+            self._export()
+        return self._h
 
     def __int__(self):
         return self.handle
 
     def __eq__(self, other):
         if isinstance(other, Stream):
-            return self.handle == other.handle
+            return self._h == other._h
         if isinstance(other, int):
-            return self.handle == other
+            return self._h == other
         return NotImplemented
 
     def __hash__(self):
-        return hash(self.handle)
+        return hash(self._h)
 
     def __cuda_stream__(self):
         return (0, self.handle)
 
     def __repr__(self):
-        if self.handle == 0:
+        if self._h == 0:
             return "<Default HIP stream>"
-        if self.handle == HIP_STREAM_PER_THREAD:
+        if self._h == HIP_STREAM_PER_THREAD:
             return "<Per-thread default HIP stream>"
         if self.external:
-            return "<External HIP stream %d>" % self.handle
-        return "<HIP stream %d>" % self.handle
+            return "<External HIP stream %d>" % self._h
+        return "<HIP stream %d>" % self._h
 
     def synchronize(self):
-        driver.nbh_stream_synchronize(self.handle or None)
+        driver.nbh_stream_synchronize(self._h or None)
 
     def query(self):
-        return _query(driver.lib.nbh_stream_query(self.handle or None), "nbh_stream_query")
+        return _query(driver.lib.nbh_stream_query(self._h or None), "nbh_stream_query")
 
     def auto_synchronize(self):
         return _SyncOnExit(self)
@@ -1369,7 +1391,7 @@ class Stream:
         slot.append(thunk)
         _pending_thunks[id(slot)] = (thunk, slot)
         try:
-            driver.nbh_stream_add_callback(self.handle or None, thunk, None)
+            driver.nbh_stream_add_callback(self._h or None, thunk, None)
         except Exception:
             _pending_thunks.pop(id(slot), None)
             raise
@@ -1449,7 +1471,7 @@ def _stream_handle(stream):
     """0 or a Stream object (or anything with __cuda_stream__) -> raw handle
     (reference :2767-2789)."""
     if isinstance(stream, Stream):
-        return stream.handle
+        return stream._h
     if isinstance(stream, int) and stream == 0:
         return 0
     protocol = getattr(stream, "__cuda_stream__", None)

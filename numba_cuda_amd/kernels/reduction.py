@@ -309,7 +309,7 @@ class Reduce:
                 arr, _ = devicearray.auto_device(arr, stream=stream)
             in_ptr = arr.device_ctypes_pointer.value
 
-        hstream = stream.handle if stream.__class__ is _Stream else _driver._stream_handle(stream)
+        hstream = stream._h if stream.__class__ is _Stream else _driver._stream_handle(stream)
         scratch = ctx._scratch.get(hstream)
         if scratch is None or hstream == _PER_THREAD:
             scratch = ctx.reduce_scratch(hstream)

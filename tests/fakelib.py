@@ -245,6 +245,9 @@ class FakeLib:
         self._next_handle += 0x10
         return self._next_handle
 
+    def nbh_stream_pin_direct(self, s):
+        return 0
+
     def nbh_stream_create(self, out):
         h = self._handle()
         self.live_streams.add(h)

@@ -19,6 +19,7 @@
 #include <unistd.h>
 extern "C" int nbh_launch_threads(int enable);
 extern "C" int nbh_launch_threads_wait(nbh_stream_t stream);
+extern "C" int nbh_stream_pin_direct(nbh_stream_t stream);
 extern "C" int nbh_reduce_queued(int op, int dtype, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                                  void *scratch, size_t scratch_bytes, nbh_stream_t stream);
 static std::mutex g_m;
@@ -84,6 +85,34 @@ int main()
     nbh_reduce_queued(0, 2, &dummy_in, 3, 6, &init, &o, &scratch, 4, streams[0]);
     nbh_queue_drain(streams[0]);
     if (nbh_queue_take_status(streams[0]) != 1 || nbh_queue_take_status(streams[0]) != 0) { printf("status\n"); return 1; }
+    // A stream whose handle leaves the library: what is queued is launched before the call returns,
+    // later launches are made by the caller (their result is there when the call returns), also
+    // for a stream that is pinned before it was ever used
+    {
+        void *st = (void *)(uintptr_t)0x5000, *fresh = (void *)(uintptr_t)0x5100;
+        std::vector<int64_t> got(200, -1);
+        for (int i = 0; i < 200; ++i) nbh_reduce_queued(0, 2, &dummy_in, i + 1, 4, &init, &got[i], &scratch, 4, st);
+        nbh_stream_pin_direct(st);
+        for (int i = 0; i < 200; ++i) if (got[i] != i + 1) { printf("pin returned before launch %d\n", i); return 1; }
+        int64_t now = -1;
+        nbh_reduce_queued(0, 2, &dummy_in, 77, 4, &init, &now, &scratch, 4, st);
+        if (now != 77) { printf("pinned stream still queues\n"); return 1; }
+        nbh_stream_pin_direct(fresh);
+        now = -1;
+        nbh_reduce_queued(0, 2, &dummy_in, 78, 4, &init, &now, &scratch, 4, fresh);
+        if (now != 78) { printf("stream pinned before use still queues\n"); return 1; }
+        nbh_queue_forget(st);
+        nbh_queue_forget(fresh);
+        // the handle value comes back for a new stream: queued again
+        now = -1;
+        g_block.store(true);
+        nbh_reduce_queued(0, 2, &dummy_in, 79, 4, &init, &now, &scratch, 4, st);
+        const bool was_queued = now == -1;
+        g_block.store(false);
+        nbh_queue_drain(st);
+        if (!was_queued || now != 79) { printf("a new stream with an old handle value is not queued\n"); return 1; }
+        nbh_queue_forget(st);
+    }
     // A fork while launches are queued: the child has no launching threads; every call that waits
     // for queues must return there, and launches go straight through (feature off in the child).
     g_block.store(true);

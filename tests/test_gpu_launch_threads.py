@@ -1,6 +1,7 @@
-"""Launching threads (kernels/reduction.py launch_threads, nbh_reduce_queued): the opt-in mode in
-which `Reduce(...)(arr, res=..., stream=s)` hands its kernel launch to a thread that belongs
-to the stream.  Results and ordering must be those of the default mode whatever else the
+"""Launching threads (kernels/reduction.py launch_threads, nbh_reduce_queued): the mode (on unless
+NUMBA_CUDA_REDUCE_LAUNCH_THREADS=0) in which `Reduce(...)(arr, res=..., stream=s)` hands its kernel
+launch to a thread that belongs to the stream, until the stream's handle is read by code outside
+the package.  Results and ordering must be those of the default mode whatever else the
 package does with the stream in between; integer data, so every comparison is exact."""
 import ctypes
 import threading
@@ -24,10 +25,7 @@ def _say(*a):
 @pytest.fixture
 def queued():
     reduction.launch_threads(True)
-    try:
-        yield
-    finally:
-        reduction.launch_threads(False)
+    yield
 
 
 def test_switching_changes_the_entry_the_native_passage_calls():
@@ -35,12 +33,12 @@ def test_switching_changes_the_entry_the_native_passage_calls():
     lib = drv.driver.lib
     direct = ctypes.cast(lib.nbh_reduce, ctypes.c_void_p).value
     through_queue = ctypes.cast(lib.nbh_reduce_queued, ctypes.c_void_p).value
-    reduction.launch_threads(True)
+    reduction.launch_threads(False)
     try:
-        assert lib._reduce_entry == through_queue
+        assert lib._reduce_entry == direct
     finally:
-        reduction.launch_threads(False)
-    assert lib._reduce_entry == direct
+        reduction.launch_threads(True)
+    assert lib._reduce_entry == through_queue
 
 
 def test_rows_over_four_streams_match_numpy(queued):
@@ -149,14 +147,14 @@ def test_a_launch_that_fails_is_reported_by_the_next_synchronize(queued):
     s = cuda.stream()
     d = cuda.to_device(np.arange(64, dtype=np.int32))
     res = cuda.device_array(1, np.int32)
-    scratch = ctx.reduce_scratch(s.handle)
+    scratch = ctx.reduce_scratch(s._h)              # `_h`: reading `handle` would take the stream out of the mode
     init = np.zeros(1, np.int32)
     # a stride that is no multiple of the item size: refused by the launch itself
     rc = lib.nbh_reduce_queued(0, 2, d.device_ctypes_pointer.value, 8, 6, init.ctypes.data,
-                               res.device_ctypes_pointer.value, scratch[0], scratch[1], s.handle)
+                               res.device_ctypes_pointer.value, scratch[0], scratch[1], s._h)
     assert rc == 0                                              # queued, not yet looked at
-    assert lib.nbh_stream_synchronize(s.handle) == 1            # hipErrorInvalidValue, reported once
-    assert lib.nbh_stream_synchronize(s.handle) == 0
+    assert lib.nbh_stream_synchronize(s._h) == 1                # hipErrorInvalidValue, reported once
+    assert lib.nbh_stream_synchronize(s._h) == 0
     sum_reduce(d, res=res, stream=s)                            # the stream is as good as before
     s.synchronize()
     assert res.copy_to_host()[0] == 64 * 63 // 2
@@ -185,7 +183,7 @@ def test_switching_back_and_forth_between_calls():
                 streams[rep % 3] = cuda.stream()     # the old one goes with its thread
             assert (out.copy_to_host() == host.sum(axis=1)).all(), rep
     finally:
-        reduction.launch_threads(False)
+        reduction.launch_threads(True)
 
 
 def test_exported_array_interface_waits_for_the_queues(queued):
@@ -203,6 +201,66 @@ def test_exported_array_interface_waits_for_the_queues(queued):
     t = torch.as_tensor(res, device="cuda")          # reads the interface
     torch.cuda.synchronize()
     assert bool((t == int(host.sum())).all())
+
+
+def test_a_stream_that_leaves_the_package_is_launched_directly_from_then_on(queued):
+    """Work queued before the handle is read is in the stream when the read returns; afterwards the
+    stream's reductions are launched by the caller (a failing launch reports at the call, not at the
+    next synchronize); a consumer of the array interface that carries the stream finds it in order."""
+    lib = drv.driver.lib
+    ctx = cuda.current_context()
+    s = cuda.stream()
+    host = np.arange(1, 200_001, dtype=np.int64)
+    d = cuda.to_device(host, stream=s)
+    res = cuda.device_array(300, np.int64, stream=s)
+    for k in range(300):
+        sum_reduce(d, res=res[k:k + 1], init=k, stream=s)
+    raw = int(s)                                      # the handle leaves: everything queued is launched
+    assert lib.nbh_stream_synchronize(raw) == 0
+    assert (res.copy_to_host(stream=s) == host.sum() + np.arange(300)).all()
+    # direct from now on: a launch the runtime refuses is reported by the call itself
+    scratch = ctx.reduce_scratch(raw)
+    init = np.zeros(1, np.int64)
+    rc = lib.nbh_reduce_queued(0, 3, d.device_ctypes_pointer.value, 8, 6, init.ctypes.data,
+                               res.device_ctypes_pointer.value, scratch[0], scratch[1], raw)
+    assert rc != 0
+    for k in range(300):
+        sum_reduce(d, res=res[k:k + 1], init=-k, stream=s)
+    s.synchronize()
+    assert (res.copy_to_host() == host.sum() - np.arange(300)).all()
+    # a stream seen first through the array interface of an array bound to it
+    torch = pytest.importorskip("torch")
+    if not torch.cuda.is_available():
+        pytest.skip("torch sees no GPU")
+    s2 = cuda.stream()
+    res2 = cuda.device_array(200, np.int64, stream=s2)
+    for k in range(200):
+        sum_reduce(d, res=res2[k:k + 1], init=7, stream=s2)
+    desc = res2.__cuda_array_interface__
+    assert desc["stream"] == s2._h and s2._exported
+    t = torch.as_tensor(res2, device="cuda")
+    torch.cuda.synchronize()
+    assert bool((t == int(host.sum()) + 7).all())
+
+
+def test_environment_variable_zero_switches_the_mode_off():
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import ctypes, numpy as np, numba_cuda_amd as cuda\n"
+        "from numba_cuda_amd.cudadrv import driver as drv\n"
+        "red = cuda.Reduce(lambda a, b: a + b)\n"
+        "h = np.arange(1000, dtype=np.int64); d = cuda.to_device(h); out = cuda.device_array(1, np.int64)\n"
+        "s = cuda.stream(); red(d, res=out, stream=s); s.synchronize()\n"
+        "lib = drv.driver.lib\n"
+        "assert lib._reduce_entry == ctypes.cast(lib.nbh_reduce, ctypes.c_void_p).value\n"
+        "assert out.copy_to_host()[0] == h.sum()\n"
+        "print('ok')\n")
+    env = dict(os.environ, NUMBA_CUDA_REDUCE_LAUNCH_THREADS="0",
+               PYTHONPATH=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    done = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert done.returncode == 0 and done.stdout.strip().endswith("ok"), done.stderr[-2000:]
 
 
 def test_environment_variable_starts_the_mode():

@@ -74,7 +74,7 @@ class _Arr:
 
 class _Stream:
     def __init__(self, handle):
-        self.handle = handle
+        self._h = handle
 
 
 class _Ctx:

@@ -211,12 +211,35 @@ def test_launch_threads_switch_needs_a_library_that_has_them(monkeypatch):
 
 def test_launch_threads_flag_is_read_from_the_environment(monkeypatch):
     from numba_cuda_amd.core import config
-    assert config.CUDA_REDUCE_LAUNCH_THREADS == 0
-    monkeypatch.setenv("NUMBA_CUDA_REDUCE_LAUNCH_THREADS", "1")
+    assert config.CUDA_REDUCE_LAUNCH_THREADS == 1          # on unless switched off
+    monkeypatch.setenv("NUMBA_CUDA_REDUCE_LAUNCH_THREADS", "0")
     config.reload_config()
     try:
-        assert config.CUDA_REDUCE_LAUNCH_THREADS == 1
+        assert config.CUDA_REDUCE_LAUNCH_THREADS == 0
     finally:
         monkeypatch.delenv("NUMBA_CUDA_REDUCE_LAUNCH_THREADS")
         config.reload_config()
-    assert config.CUDA_REDUCE_LAUNCH_THREADS == 0
+    assert config.CUDA_REDUCE_LAUNCH_THREADS == 1
+
+
+def test_reading_the_handle_hands_the_stream_out_of_the_package(fake_gpu):
+    """`handle`, int() and __cuda_stream__ are how a stream leaves the package: the library is told
+    once (nbh_stream_pin_direct), so that nothing stays queued for a stream foreign code may use.
+    External streams are told at creation; the default streams never are; `_h` tells nobody."""
+    pinned = []
+    fake_gpu.nbh_stream_pin_direct = lambda s: pinned.append(s) or 0
+    s = cuda.stream()
+    assert s._h and not s._exported and pinned == []
+    assert drv._stream_handle(s) == s._h and pinned == []          # the package's own way to the handle
+    assert s.handle == s._h and pinned == [s._h]
+    assert int(s) == s._h and s.__cuda_stream__() == (0, s._h) and pinned == [s._h]   # told once
+    t = cuda.stream()
+    assert int(t) == t._h and pinned[-1] == t._h
+    u = cuda.stream()
+    d = cuda.device_array(4, np.float32, stream=u)
+    assert d.__cuda_array_interface__["stream"] == u._h and pinned[-1] == u._h
+    ext = cuda.external_stream(0x7700)
+    assert pinned[-1] == 0x7700 and ext.external
+    before = list(pinned)
+    assert cuda.default_stream().handle == 0 and cuda.per_thread_default_stream().handle == 2
+    assert pinned == before
