@@ -333,14 +333,99 @@ __device__ __forceinline__ void apply_lut(const u64x2_t *__restrict__ lut, uint6
 constexpr int kTabBlock = 1024;
 constexpr int64_t kTablesFrom = 1 << 18;  // below this the table load outweighs its benefit
 
+// One application of J^64 to every lane's own state, 16 look-ups of 8 bits each, WITHOUT bank
+// conflicts.  A wavefront's lanes hold unrelated states, so look-ups into one table hit random
+// banks: measured, 61 % of the LDS's active cycles were conflict stalls.  The banks repeat
+// every 256 bytes and a 128-bit read takes four of them, so the tables are laid out
+// [value][position]: row v (256 bytes) holds the 16 entries that value v selects, position p
+// in banks 4p .. 4p+3.  In look-up round t lane l takes position p = t XOR (l mod 16): over
+// the 16 rounds every lane visits every position, and in any one round the 16 lanes of a row
+// of the wavefront read 16 different positions - 16 different groups of banks, whatever the
+// values.  Which byte of the state a lane needs in round t then depends on the lane; the state
+// is permuted once per step (bytes by a per-lane v_perm selector, words by conditional swaps) so
+// that round t finds its byte in a fixed place.
+struct LaneOrder {
+    uint32_t byte_select;  // v_perm selector: byte i of the result is byte i ^ (l & 3) of the source
+    bool swap1, swap2;     // exchange words 0<->1, 2<->3 / 0<->2, 1<->3 of the 128-bit state
+    uint32_t base;         // (l mod 16) * 16: this lane's position in round 0, as a byte offset in a table row
+};
+
+__device__ __forceinline__ LaneOrder lane_order(int lane)
+{
+    const uint32_t l16 = (uint32_t)lane & 15u;
+    LaneOrder o;
+    o.byte_select = 0x03020100u ^ ((l16 & 3u) * 0x01010101u);
+    o.swap1 = (l16 & 4u) != 0;
+    o.swap2 = (l16 & 8u) != 0;
+    o.base = l16 << 4;
+    return o;
+}
+
+__device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c)
+{
+    return (uint32_t)__builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+}
+
+// lut8: the J^64 table in LDS as [256 values][16 positions] of 16-byte entries
+__device__ __forceinline__ void apply_lut8_spread(const unsigned char *__restrict__ lut8, const LaneOrder &o,
+                                                  uint64_t &s0, uint64_t &s1)
+{
+    uint32_t d0 = (uint32_t)s0, d1 = (uint32_t)(s0 >> 32), d2 = (uint32_t)s1, d3 = (uint32_t)(s1 >> 32);
+    // word j of the permuted state is word j ^ (l16 >> 2) of the state ...
+    uint32_t e0 = o.swap1 ? d1 : d0, e1 = o.swap1 ? d0 : d1, e2 = o.swap1 ? d3 : d2, e3 = o.swap1 ? d2 : d3;
+    uint32_t r[4];
+    r[0] = o.swap2 ? e2 : e0;
+    r[1] = o.swap2 ? e3 : e1;
+    r[2] = o.swap2 ? e0 : e2;
+    r[3] = o.swap2 ? e1 : e3;
+    // ... with its bytes exchanged the same way
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        r[j] = __builtin_amdgcn_perm(r[j], r[j], o.byte_select);
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    u32x4_t got[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        const uint32_t w = r[t >> 2];
+        const int k = t & 3;
+        // (byte k of w) << 8: the row of the table
+        const uint32_t row = k == 0 ? (w << 8) : k == 1 ? w : k == 2 ? (w >> 8) : (w >> 16);
+        const uint32_t at = (row & 0xFF00u) | (o.base ^ (uint32_t)(t << 4));
+        got[t] = *reinterpret_cast<const u32x4_t *>(lut8 + at);
+    }
+    uint32_t acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        uint32_t a = xor3(got[0][c], got[1][c], got[2][c]);
+        a = xor3(a, got[3][c], got[4][c]);
+        a = xor3(a, got[5][c], got[6][c]);
+        a = xor3(a, got[7][c], got[8][c]);
+        a = xor3(a, got[9][c], got[10][c]);
+        a = xor3(a, got[11][c], got[12][c]);
+        a = xor3(a, got[13][c], got[14][c]);
+        acc[c] = a ^ got[15][c];
+    }
+    s0 = ((uint64_t)acc[1] << 32) | acc[0];
+    s1 = ((uint64_t)acc[3] << 32) | acc[2];
+}
+
 __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t *__restrict__ states, int64_t n,
                                                                        uint64_t b0, uint64_t b1,
                                                                        const U128 *__restrict__ table,
                                                                        const u64x2_t *__restrict__ lut_global)
 {
-    __shared__ u64x2_t lut[kLutEntries];  // 112 KiB: lut4[6][32][16] then lut8[16][256]
-    for (int i = threadIdx.x; i < kLutEntries; i += kTabBlock)
-        lut[i] = lut_global[i];
+    // 112 KiB: lut4[6][32][16] as it comes, then lut8 transposed to [256 values][16 positions]
+    __shared__ u64x2_t lut[kLutEntries];
+    constexpr int kLut4 = kLaneTables * 32 * 16;
+    for (int i = threadIdx.x; i < kLutEntries; i += kTabBlock) {
+        const u64x2_t v = lut_global[i];
+        if (i < kLut4) {
+            lut[i] = v;
+        } else {
+            const int j = i - kLut4;  // lut8[p][value] in global memory
+            lut[kLut4 + (j & 255) * 16 + (j >> 8)] = v;
+        }
+    }
     __syncthreads();
 
     const int lane = threadIdx.x & 63;
@@ -357,7 +442,8 @@ __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t 
     for (int k = 0; k < kLaneTables; ++k)
         if ((lane >> k) & 1)
             apply_lut<4>(lut + k * 32 * 16, s0, s1);
-    const u64x2_t *__restrict__ step = lut + kLaneTables * 32 * 16;  // J^64, 8 bits per lookup
+    const unsigned char *__restrict__ step = reinterpret_cast<const unsigned char *>(lut + kLut4);  // J^64
+    const LaneOrder order = lane_order(lane);
     for (int g = 0; g < kInitSteps; ++g) {
         if (first + (int64_t)g * 64 >= n)
             break;
@@ -367,7 +453,7 @@ __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t 
             *reinterpret_cast<u64x2_t *>(states + 2 * idx) = v;
         }
         if (g + 1 < kInitSteps)
-            apply_lut<8>(step, s0, s1);
+            apply_lut8_spread(step, order, s0, s1);
     }
 }
 
