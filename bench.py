@@ -7,13 +7,16 @@ full reduction, issued through the public API into a device result slot; inputs
 are resident in HBM before the clock starts.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others]
+                    [--view-cols N] [--elements N]
 
 Without --workload the same line carries an `others` array with every other
 benchmark configuration measured in the same process: reduce_f32_max,
 reduce_f64_sum, reduce_i64_sum, reduce_f32_functor (a translated functor),
 reduce_f32_sum_reference_order (the reference's association order), transpose_f32,
-transpose_f64, transpose_i16, rng_init, rng_uniform_f32, rng_normal_f64, batched_reduce.  --workload NAME measures
-just one of them (or copy_f32, the counter calibration kernel) as the headline.
+transpose_f64, transpose_i16, rng_init, rng_uniform_f32, rng_normal_f64, batched_reduce, and ends with
+`others_summary`, the same figures in short.  --workload NAME measures just one of them (or copy_f32, the counter
+calibration kernel) as the headline; --view-cols N (transposes: the first N columns only, pitches unchanged) and
+--elements N (copy_f32) give the time-against-size tables of profiles/.
 """
 
 import argparse
@@ -34,27 +37,20 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E published peak
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (see profiles/); filled in per workload once measured, else None
 MEASURED_TRAFFIC = {
-    # profiles/reduce_kernel_f32_sum_2p28.txt: 1 073 783 602 B fetched + 32 821 B written
-    "reduce_f32_sum": 1073816423,
-    # profiles/copy_flat_f32_2p28.txt: the calibration kernel itself
-    "copy_f32": 2147483648,
-    # profiles/transpose_packets_f32_16384sq.txt: 1 073 761 075 B fetched + 1 074 512 910 B written
-    "transpose_f32": 2148273985,
-    # profiles/xoroshiro_fill_and_init_2p24.txt: 268 618 773 B fetched + 4 563 547 721 B written
-    "rng_uniform_f32": 4832166494,
-    # profiles/transpose_sheared_f64_12345x6789.txt: 768 287 439 B fetched + 670 489 125 B written
-    "transpose_f64": 1438776564,
-    # profiles/hbm_counters_other_workloads.txt
-    "reduce_f32_max": 1073827256,
-    "reduce_f64_sum": 1073823652,
-    "reduce_i64_sum": 2147537460,
-    "transpose_i16": 1073901040,      # profiles/transpose_packets_f32_16384sq.txt, last section
-    # profiles/reduce_ordered_kernel_f32_sum_2p28.txt: 1 073 919 663 B fetched + 16 441 B written
-    "reduce_f32_sum_reference_order": 1073936104,
-    # profiles/reduce_kernel_other_dtypes_and_batched.txt: 1 073 905 148 B fetched + 32 821 B written
-    "reduce_f32_functor": 1073937969,
-    "rng_normal_f64": 2684437180,
-    "rng_init": 269594109,
+    # fetched + written bytes per launch; each figure is derived in the profiles/ file TRAFFIC_SOURCE names
+    "reduce_f32_sum": 1073804215,
+    "copy_f32": 2147483648,                      # the calibration kernel itself
+    "transpose_f32": 2148246600,
+    "transpose_f64": 1438988253,
+    "transpose_i16": 1073881556,
+    "reduce_f32_max": 1073819617,
+    "reduce_f64_sum": 1073818517,
+    "reduce_i64_sum": 2147532373,
+    "reduce_f32_sum_reference_order": 1073945113,
+    "reduce_f32_functor": 1073931926,
+    "rng_uniform_f32": 4831464874,
+    "rng_normal_f64": 2684020932,
+    "rng_init": 269598301,
 }
 
 
@@ -89,8 +85,7 @@ def _cpu_baseline_reduce(a_host, target_seconds=12.0, functor=lambda x, y: x + y
     red(sample, init=0)
     dt = time.perf_counter() - t0
     return {"value": round(sample.nbytes / dt / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "first 2^%d %s elements of the same input, simulator-style left fold "
-                      "(functools.reduce over NumPy scalars), %.1f s" % (n.bit_length() - 1, a_host.dtype.name, dt),
+            "sample": "left fold over the first 2^%d %s elements, %.1f s" % (n.bit_length() - 1, a_host.dtype.name, dt),
             "elements_per_s": round(n / dt, 1), "host_cores_available": os.cpu_count()}
 
 
@@ -106,8 +101,7 @@ def _cpu_baseline_transpose(shape, dtype):
         reps += 1
     dt = (time.perf_counter() - t0) / reps
     return {"value": round(2 * a.nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "256 x 256 %s, simulator transpose (NumPy view) + materialising copy, %d repetitions"
-                      % (np.dtype(dtype).name, reps),
+            "sample": "256 x 256 %s view + copy, %d repetitions" % (np.dtype(dtype).name, reps),
             "host_cores_available": os.cpu_count()}
 
 
@@ -124,7 +118,7 @@ def _cpu_baseline_rng(name, nthreads=4096):
     t_init = time.perf_counter() - t0
     if name == "rng_init":
         return {"value": round(16 * nthreads / t_init / 1e9, 9), "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": "%d states by the sequential jump chain in NumPy-scalar Python, %.1f s" % (nthreads, t_init),
+                "sample": "%d states, sequential jump chain, %.1f s" % (nthreads, t_init),
                 "states_per_s": round(nthreads / t_init, 1), "host_cores_available": os.cpu_count()}
     draw, count, size = ((sim.uniform_float32, 64, 4) if name == "rng_uniform_f32" else (sim.normal_float64, 16, 8))
     t0 = time.perf_counter()
@@ -133,8 +127,7 @@ def _cpu_baseline_rng(name, nthreads=4096):
             draw(states, t)
     dt = time.perf_counter() - t0
     return {"value": round(size * nthreads * count / dt / 1e9, 9), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "%d generators x %d draws in NumPy-scalar Python, %.1f s (state initialisation %.1f s not included)"
-                      % (nthreads, count, dt, t_init),
+            "sample": "%d generators x %d draws, %.1f s (+ %.1f s state init)" % (nthreads, count, dt, t_init),
             "outputs_per_s": round(nthreads * count / dt, 1), "host_cores_available": os.cpu_count()}
 
 
@@ -142,8 +135,10 @@ def _hypot(a, b):
     return math.sqrt(a * a + b * b)
 
 
-def _workload(name, cuda):
-    """-> dict(desc, dtype, algo_bytes, units, step(i), stream, host_input, kernel)"""
+def _workload(name, cuda, options):
+    """-> dict(desc, dtype, algo_bytes, units, step(i), stream, host_input, kernel).  `options`:
+    view_cols (transposes: only the first N columns of the matrix, a view with the full
+    matrix's row pitches on both sides) and elements (copy_f32: another size)."""
     from numba_cuda_amd import random as nrandom
     from numba_cuda_amd.kernels.transpose import transpose
     stream = cuda.stream()
@@ -176,13 +171,14 @@ def _workload(name, cuda):
         res = cuda.device_array(1, dtype=host.dtype)
         red = mx if name.endswith("max") else add
         init = -np.inf if name.endswith("max") else 0
-        kernel = "reduce_kernel"
+        ctype = {"float32": "float", "float64": "double", "int64": "long"}[host.dtype.name]
+        kernel = "reduce_kernel<%s, (anonymous namespace)::%s, false>" % (ctype, "OpMax" if name.endswith("max") else "OpAdd")
         if name.endswith("functor"):
             red = cuda.Reduce(_hypot)
             kernel = "nbh_custom_reduce"
         if name.endswith("reference_order"):
             red = cuda.Reduce(lambda a, b: a + b, reference_order=True)
-            kernel = "reduce_ordered_kernel"
+            kernel = "reduce_ordered_kernel<float, (anonymous namespace)::OpAdd, true>"
 
         def step(i):
             red(bufs[i & 1], res=res, init=init, stream=stream)
@@ -202,15 +198,27 @@ def _workload(name, cuda):
             raise SystemExit("unknown workload %s" % name)
         src = cuda.to_device(host).bind(stream)
         dst = cuda.device_array((host.shape[1], host.shape[0]), dtype=host.dtype, stream=stream)
+        desc = "transpose %s %dx%d, seed 2" % (host.dtype.name, host.shape[0], host.shape[1])
+        moved, items = 2 * host.nbytes, host.size
+        view_cols = options.get("view_cols")
+        if view_cols:
+            # the first columns only, both arrays keeping their pitches: how the time grows with
+            # the size of the matrix while everything else stays what it is
+            view_cols = min(int(view_cols), host.shape[1])
+            src, dst = src[:, :view_cols], dst[:view_cols, :]
+            desc += ", columns 0..%d only (row pitches unchanged)" % view_cols
+            items = host.shape[0] * view_cols
+            moved = 2 * items * host.dtype.itemsize
 
         def step(i):
             transpose(src, dst)
 
-        return dict(desc="transpose %s %dx%d, seed 2" % (host.dtype.name, host.shape[0], host.shape[1]),
-                    dtype=host.dtype.name, algo_bytes=2 * host.nbytes, units=host.size, step=step,
+        return dict(desc=desc,
+                    dtype=host.dtype.name, algo_bytes=moved, units=items, step=step,
                     stream=stream, host=None, keep=(src, dst),
-                    kernel={"transpose_f32": "transpose_packets<4, true>", "transpose_f64": "transpose_sheared<RingCfg<8, 128, 32, 4, 256, 1>>",
-                            "transpose_i16": "transpose_packets<2, true>"}[name])
+                    kernel={"transpose_f32": "transpose_packets<4, true, (anonymous namespace)::ShapeOf<4> >",
+                            "transpose_f64": "transpose_sheared<(anonymous namespace)::RingCfg<8, 128, 32, 4, 256, 1, 128> >",
+                            "transpose_i16": "transpose_packets<2, true, (anonymous namespace)::ShapeOf<2> >"}[name])
     if name.startswith("rng_"):
         n = 2**24
         states = cuda.device_array(n, dtype=nrandom.xoroshiro128p_dtype)
@@ -228,7 +236,7 @@ def _workload(name, cuda):
                 nrandom.xoroshiro128p_fill(states, out, 64, nrandom.UNIFORM, stream)
             return dict(desc="xoroshiro128p 2^24 generators x 64 uniform float32", dtype="u64",
                         algo_bytes=4 * n * 64 + 32 * n, units=n * 64, step=step, stream=stream, host=None,
-                        kernel="fill_regs_kernel<UniformF32>", keep=(states, out))
+                        kernel="fill_regs_kernel<(anonymous namespace)::UniformF32>", keep=(states, out))
         if name == "rng_normal_f64":
             out = cuda.device_array(n * 16, np.float64)
 
@@ -236,11 +244,11 @@ def _workload(name, cuda):
                 nrandom.xoroshiro128p_fill(states, out, 16, nrandom.NORMAL, stream)
             return dict(desc="xoroshiro128p 2^24 generators x 16 normal float64", dtype="f64",
                         algo_bytes=8 * n * 16 + 32 * n, units=n * 16, step=step, stream=stream, host=None,
-                        kernel="fill_kernel<NormalF64>", keep=(states, out))
+                        kernel="fill_kernel<(anonymous namespace)::NormalF64, true, 1>", keep=(states, out))
     if name == "copy_f32":
         # flat device-to-device assignment: the plain copy kernel of known size that
         # the rocprofv3 FETCH_SIZE / WRITE_SIZE counters are calibrated against
-        host = np.random.default_rng(4).random(2**28, dtype=np.float32)
+        host = np.random.default_rng(4).random(int(options.get("elements") or 2**28), dtype=np.float32)
         src = cuda.to_device(host)
         dst = cuda.device_array_like(host)
         everything = slice(None)
@@ -248,9 +256,9 @@ def _workload(name, cuda):
         def step(i):
             dst.setitem(everything, src, stream=stream)
 
-        return dict(desc="flat copy dst[:] = src, 2^28 float32 (counter calibration)", dtype="u8",
+        return dict(desc="flat copy dst[:] = src, %d float32 (counter calibration)" % host.size, dtype="u8",
                     algo_bytes=2 * host.nbytes, units=host.size, step=step, stream=stream, host=None,
-                    kernel="copy_flat", keep=(src, dst))
+                    kernel="copy_flat<4>", keep=(src, dst))
     if name == "batched_reduce":
         rows, cols = 4096, 65536
         host = np.random.default_rng(3).uniform(-1, 1, (rows, cols)).astype(np.float32)
@@ -311,7 +319,8 @@ def _workload(name, cuda):
 
         return dict(desc="4096 x (65536 fp32) row sums round-robin over 4 streams, seed 3", dtype="f32",
                     algo_bytes=host.nbytes, units=rows, step=step, stream=streams[0], host=host,
-                    kernel="reduce_kernel", keep=(dm, out, streams, views, slots), calls_per_step=rows,
+                    kernel="reduce_kernel<float, (anonymous namespace)::OpAdd, false>", keep=(dm, out, streams, views, slots),
+                    calls_per_step=rows,
                     extras=extras)
     raise SystemExit("unknown workload %s" % name)
 
@@ -320,16 +329,16 @@ TRAFFIC_SOURCE = {
     "reduce_f32_sum": "profiles/reduce_kernel_f32_sum_2p28.txt",
     "copy_f32": "profiles/copy_flat_f32_2p28.txt",
     "transpose_f32": "profiles/transpose_packets_f32_16384sq.txt",
-    "rng_uniform_f32": "profiles/xoroshiro_fill_and_init_2p24.txt",
-    "transpose_f64": "profiles/transpose_sheared_f64_12345x6789.txt",
-    "reduce_f32_max": "profiles/hbm_counters_other_workloads.txt",
-    "reduce_f64_sum": "profiles/hbm_counters_other_workloads.txt",
-    "reduce_i64_sum": "profiles/hbm_counters_other_workloads.txt",
     "transpose_i16": "profiles/transpose_packets_f32_16384sq.txt",
-    "reduce_f32_sum_reference_order": "profiles/reduce_ordered_kernel_f32_sum_2p28.txt",
+    "transpose_f64": "profiles/transpose_sheared_f64_12345x6789.txt",
+    "reduce_f32_max": "profiles/reduce_kernel_other_dtypes_and_batched.txt",
+    "reduce_f64_sum": "profiles/reduce_kernel_other_dtypes_and_batched.txt",
+    "reduce_i64_sum": "profiles/reduce_kernel_other_dtypes_and_batched.txt",
     "reduce_f32_functor": "profiles/reduce_kernel_other_dtypes_and_batched.txt",
-    "rng_normal_f64": "profiles/hbm_counters_other_workloads.txt",
-    "rng_init": "profiles/hbm_counters_other_workloads.txt",
+    "reduce_f32_sum_reference_order": "profiles/reduce_ordered_kernel_f32_sum_2p28.txt",
+    "rng_init": "profiles/xoroshiro_fill_and_init_2p24.txt",
+    "rng_uniform_f32": "profiles/xoroshiro_fill_and_init_2p24.txt",
+    "rng_normal_f64": "profiles/xoroshiro_fill_and_init_2p24.txt",
 }
 
 OTHER_WORKLOADS = ["reduce_f32_max", "reduce_f64_sum", "reduce_i64_sum", "reduce_f32_functor", "reduce_f32_sum_reference_order",
@@ -352,17 +361,34 @@ def _cpu_baseline(name, w, seconds):
     return None
 
 
-def measure(cuda, name, steps, warmup, cpu_seconds):
+# Workloads whose kernels run long enough and hot enough for the device's power management to
+# show: the first launches after an idle spell run fast, the next ones are throttled (up to
+# 40 % on the arithmetic-heavy generators) and it takes some fifty launches to settle.  For
+# these the line carries both figures: `first10_us_avg`, the ten launches that follow the
+# driver's own --warmup, and the settled one (after SETTLE_LAUNCHES more untimed launches),
+# which `value` and `roofline` are.
+POWER_MANAGED = ("rng_uniform_f32", "rng_normal_f64", "reduce_f32_functor", "reduce_f32_sum_reference_order")
+SETTLE_LAUNCHES = 50
+
+
+def measure(cuda, name, steps, warmup, cpu_seconds, options=None):
     """One workload: `warmup` untimed steps, `steps` timed ones between device-wide
     synchronisations (wall clock -> value), the same number again between a HIP
     event pair on the launch stream (-> roofline), and the CPU baseline beside it
     (cpu_seconds = 0: none)."""
-    w = _workload(name, cuda)
+    w = _workload(name, cuda, options or {})
     stream, step = w["stream"], w["step"]
     for i in range(warmup):
         step(i)
     stream.synchronize()
     cuda.synchronize()
+    first10 = None
+    if name in POWER_MANAGED:
+        first10 = _event_timed_launches(cuda, stream, step, 10) * 1e3
+        for i in range(SETTLE_LAUNCHES):
+            step(i)
+        stream.synchronize()
+        cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
         step(i)
@@ -383,6 +409,11 @@ def measure(cuda, name, steps, warmup, cpu_seconds):
                     "traffic_source": TRAFFIC_SOURCE.get(name),
                     "kernel": w["kernel"], "algorithmic_bytes_per_launch": w["algo_bytes"],
                     "launch_us_avg": round(launch_ms * 1e3, 2), "launches_timed": steps}
+        if first10 is not None:
+            roofline["first10_us_avg"] = round(first10, 2)
+            roofline["settle_launches"] = SETTLE_LAUNCHES
+        if options:
+            roofline["traffic"] = None          # a view or another size than the counters were taken on
     cpu = _cpu_baseline(name, w, cpu_seconds) if cpu_seconds > 0 else None
     out = {"name": name, "workload": w["desc"], "dtype": w["dtype"], "value": round(gbs, 1), "unit": "GB/s",
            "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 5),
@@ -412,6 +443,9 @@ def main():
     ap.add_argument("--workload", default=None,
                     help="measure only this workload (default: the headline workload, then every other "
                          "configuration in an `others` array)")
+    ap.add_argument("--view-cols", type=int, default=None,
+                    help="transpose workloads: only the first N columns of the matrix (a view; pitches unchanged)")
+    ap.add_argument("--elements", type=int, default=None, help="copy_f32: number of float32 items")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true")
     args = ap.parse_args()
@@ -424,7 +458,8 @@ def main():
         raise SystemExit("no GPU / HIP library: %s" % cuda.cuda_error())
 
     name = args.workload or "reduce_f32_sum"
-    head = measure(cuda, name, args.steps, args.warmup, 0 if args.no_cpu_baseline else 12.0)
+    options = {k: v for k, v in (("view_cols", args.view_cols), ("elements", args.elements)) if v}
+    head = measure(cuda, name, args.steps, args.warmup, 0 if args.no_cpu_baseline else 12.0, options)
     line = {
         "metric": "achieved HBM GB/s (% of 8 TB/s) for cuda.reduce fp32 sum at 2^28 elems"
         if name == "reduce_f32_sum" else "achieved HBM GB/s for " + name,
@@ -446,14 +481,14 @@ def main():
         for other in OTHER_WORKLOADS:
             _release_device_memory(cuda)
             steps, warmup = (10, 2) if other == "batched_reduce" else (min(args.steps, 50), min(args.warmup, 5))
-            if other in ("rng_uniform_f32", "rng_normal_f64"):
-                # millisecond-long, arithmetic-heavy launches: the device's power management lets the
-                # first three run fast, throttles the next ones by up to 40 % and takes some fifty
-                # launches to settle (profiles/xoroshiro_fill_and_init_2p24.txt); sixty untimed ones first
-                warmup = max(warmup, 60)
             print("bench: %s ..." % other, file=sys.stderr, flush=True)
             others.append(measure(cuda, other, steps, warmup, 0 if args.no_cpu_baseline else 2.0))
         line["others"] = others
+        # the same figures once more, compact and LAST on the line, so that a reader who keeps
+        # only the end of the line still has every workload: name -> [GB/s, fraction of the HBM
+        # peak by the event-timed launches (None: per-call workload), ms per step]
+        line["others_summary"] = {o["name"]: [o["value"], (o["roofline"] or {}).get("frac"), o["ms_per_step"]]
+                                  for o in [dict(head, name=name)] + others}
     print(json.dumps(line))
 
 
