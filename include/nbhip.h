@@ -248,11 +248,13 @@ int nbh_reduce_noalloc(int op, int dtype, const void *in, int64_t n, int64_t in_
  * nbh_reduce_compile builds, with the HIP run-time compiler (libhiprtc.so, loaded on
  * first use), the kernels for
  *     __device__ T nbh_op(T a, T b) { <body> }
- * where T is the C type of `dtype` (NBH_I8 .. NBH_F64 and NBH_F16; not the complex types)
- * and `body` is C++ that returns the combined value.  Available to the body: the HIP
- * device math functions, nbh_i64 / nbh_u64 (64-bit integer types), nbh_floordiv(x, y) and
- * nbh_mod(x, y) with Python's rounding for nbh_i64, nbh_u64, float and double, and
- * nbh_ipow(x, e).  Needs no device.  On failure the compiler's messages are in `log`
+ * where T is the C type of `dtype` (NBH_I8 .. NBH_F64, NBH_F16; NBH_C64 / NBH_C128 as
+ * nbh_c64 / nbh_c128, structs {re, im} of float / double) and `body` is C++ that returns
+ * the combined value.  Available to the body: the HIP device math functions, nbh_i64 /
+ * nbh_u64 (64-bit integer types), nbh_floordiv(x, y) and nbh_mod(x, y) with Python's
+ * rounding for nbh_i64, nbh_u64, float and double, nbh_ipow(x, e), and for the complex
+ * types + - * / == != as the reference's JIT lowers them (numba/cuda/cpython/numbers.py:
+ * 1091-1221), nbh_cabs(z), nbh_conj(z) and nbh_cplx_from<float | double>(x) for conversions.  Needs no device.  On failure the compiler's messages are in `log`
  * (NUL-terminated, cut to log_bytes) and the result is hipErrorInvalidSource (300), or
  * hipErrorSharedObjectInitFailed (303) when the compiler library is absent.
  * `*op` stays valid until nbh_reduce_op_free(op); it may be used from any thread and on
@@ -269,6 +271,13 @@ int nbh_reduce_op_free(void *op);
  * way: the ticket is handed back at zero).  One launch on `stream`, fully asynchronous. */
 int nbh_reduce_custom(void *op, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
                       void *scratch, size_t scratch_bytes, nbh_stream_t stream);
+
+/* The same reduction with every application of nbh_op on the same pair of values, in the
+ * same order, as a run of the reference's kernels (kernels/reduction.py:22-166 launched as
+ * in :233-258): the result then has the reference's bits also for operations that are not
+ * associative or whose rounding depends on the order.  Same arguments, one launch. */
+int nbh_reduce_custom_ordered(void *op, const void *in, int64_t n, int64_t in_stride, const void *init, void *out,
+                              void *scratch, size_t scratch_bytes, nbh_stream_t stream);
 
 /* ---- transpose ------------------------------------------------------------ */
 

@@ -76,6 +76,7 @@ SIGNATURES = {
     "nbh_reduce_op_dtype": (c_int, [c_vp]),
     "nbh_reduce_op_free": (c_int, [c_vp]),
     "nbh_reduce_custom": (c_int, [c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_size, c_vp]),
+    "nbh_reduce_custom_ordered": (c_int, [c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_size, c_vp]),
     "nbh_transpose": (c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "nbh_assign": (c_int, [c_vp, c_vp, c_int, P(c_i64), P(c_i64), P(c_i64), c_i64, c_vp]),
     "nbh_fill": (c_int, [c_vp, c_int, P(c_i64), P(c_i64), c_i64, c_vp, c_vp]),

@@ -99,15 +99,74 @@ const char *type_name(int dtype, size_t *elem)
     case NBH_F32: *elem = 4; return "float";
     case NBH_F64: *elem = 8; return "double";
     case NBH_F16: *elem = 2; return "_Float16";
+    case NBH_C64: *elem = 8; return "nbh_c64";
+    case NBH_C128: *elem = 16; return "nbh_c128";
     default: return nullptr;
     }
 }
 
-// Device source: `typedef <type> T;` goes in front, the caller's body replaces @BODY@.
+// Device source: the element type replaces @T@, the caller's body replaces @BODY@.
 const char kSource[] = R"NBHSRC(
 typedef long long nbh_i64;
 typedef unsigned long long nbh_u64;
 typedef unsigned int nbh_u32x4 __attribute__((ext_vector_type(4)));
+
+// Complex numbers as the reference's JIT computes with them (numba/cuda/cpython/numbers.py:
+// :1091-1120 sums and differences part by part, :1123-1146 the product as (ac - bd) + (ad + bc)i
+// with every product and sum rounded once, :1149-1179 the quotient by CPython's algorithm,
+// :1200-1221 equality, :1224-1233 abs as hypot).  An aggregate: it lives in unions with raw words.
+template <typename R> struct nbh_cplx { R re, im; };
+typedef nbh_cplx<float> nbh_c64;
+typedef nbh_cplx<double> nbh_c128;
+typedef @T@ T;
+
+template <typename R> __device__ __forceinline__ nbh_cplx<R> operator+(nbh_cplx<R> x, nbh_cplx<R> y)
+{
+    return {x.re + y.re, x.im + y.im};
+}
+template <typename R> __device__ __forceinline__ nbh_cplx<R> operator-(nbh_cplx<R> x, nbh_cplx<R> y)
+{
+    return {x.re - y.re, x.im - y.im};
+}
+template <typename R> __device__ __forceinline__ nbh_cplx<R> operator-(nbh_cplx<R> x) { return {-x.re, -x.im}; }
+template <typename R> __device__ __forceinline__ nbh_cplx<R> operator*(nbh_cplx<R> x, nbh_cplx<R> y)
+{
+    const R ac = x.re * y.re, bd = x.im * y.im, ad = x.re * y.im, bc = x.im * y.re;
+    return {ac - bd, ad + bc};
+}
+// a zero divisor raises ZeroDivisionError in Python; here it gives NaN + NaN i
+template <typename R> __device__ __forceinline__ nbh_cplx<R> operator/(nbh_cplx<R> x, nbh_cplx<R> y)
+{
+    const R nan = (R)__builtin_nan("");
+    const R abs_re = y.re < 0 ? -y.re : y.re, abs_im = y.im < 0 ? -y.im : y.im;
+    if (abs_re >= abs_im) {
+        if (y.re == 0)
+            return {nan, nan};
+        const R ratio = y.im / y.re, denom = y.re + y.im * ratio;
+        return {(x.re + x.im * ratio) / denom, (x.im - x.re * ratio) / denom};
+    }
+    if (y.im == 0)
+        return {nan, nan};
+    const R ratio = y.re / y.im, denom = y.re * ratio + y.im;
+    return {(x.re * ratio + x.im) / denom, (x.im * ratio - x.re) / denom};
+}
+template <typename R> __device__ __forceinline__ bool operator==(nbh_cplx<R> x, nbh_cplx<R> y)
+{
+    return x.re == y.re && x.im == y.im;
+}
+template <typename R> __device__ __forceinline__ bool operator!=(nbh_cplx<R> x, nbh_cplx<R> y)
+{
+    return x.re != y.re || x.im != y.im;
+}
+__device__ __forceinline__ float nbh_cabs(nbh_c64 z) { return hypotf(z.re, z.im); }
+__device__ __forceinline__ double nbh_cabs(nbh_c128 z) { return hypot(z.re, z.im); }
+template <typename R> __device__ __forceinline__ nbh_cplx<R> nbh_conj(nbh_cplx<R> z) { return {z.re, -z.im}; }
+// conversions into a complex type: from a real number (imaginary part 0) or the other complex type
+template <typename R, typename X> __device__ __forceinline__ nbh_cplx<R> nbh_cplx_from(X x) { return {(R)x, (R)0}; }
+template <typename R, typename Q> __device__ __forceinline__ nbh_cplx<R> nbh_cplx_from(nbh_cplx<Q> z)
+{
+    return {(R)z.re, (R)z.im};
+}
 
 // Python's // and % (round towards minus infinity, the remainder takes the divisor's
 // sign); a zero divisor gives 0 instead of raising
@@ -160,20 +219,18 @@ constexpr int kItems = 16 / (int)sizeof(T);     // elements per 16-byte packet
 constexpr int kThreads = 512, kWaves = 8, kUnroll = 4;
 constexpr long long kPiece = 2 * kThreads;      // packets per dealt piece
 union nbh_packet { nbh_u32x4 raw; T item[kItems]; };
-union nbh_slot { nbh_u64 word; T value; };
+// a value as the 64-bit words it travels in (shuffles, the partials in the scratch buffer)
+constexpr int kSlotWords = ((int)sizeof(T) + 7) / 8;
+union nbh_image { nbh_u64 w[kSlotWords]; T value; };
 
-__device__ __forceinline__ nbh_u64 nbh_word_of(T v)
+__device__ __forceinline__ nbh_image nbh_image_of(T v)
 {
-    nbh_slot s;
-    s.word = 0;
+    nbh_image s;
+#pragma unroll
+    for (int k = 0; k < kSlotWords; ++k)
+        s.w[k] = 0;
     s.value = v;
-    return s.word;
-}
-__device__ __forceinline__ T nbh_value_of(nbh_u64 w)
-{
-    nbh_slot s;
-    s.word = w;
-    return s.value;
+    return s;
 }
 __device__ __forceinline__ void nbh_take(T &acc, bool &have, T v)
 {
@@ -198,23 +255,27 @@ __device__ __forceinline__ void nbh_fold_workgroup(T &acc, bool &have)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
-        const nbh_u64 theirs = __shfl_down(nbh_word_of(acc), off, 64);
+        const nbh_image mine = nbh_image_of(acc);
+        nbh_image theirs;
+#pragma unroll
+        for (int k = 0; k < kSlotWords; ++k)
+            theirs.w[k] = __shfl_down(mine.w[k], off, 64);
         const int they_have = __shfl_down((int)have, off, 64);
         if (lane + off < 64 && they_have)
-            nbh_take(acc, have, nbh_value_of(theirs));
+            nbh_take(acc, have, theirs.value);
     }
-    __shared__ nbh_u64 wave_value[kWaves];
+    __shared__ T wave_value[kWaves];
     __shared__ int wave_has[kWaves];
     __syncthreads();  // the slots may still be read from a previous fold
     if (lane == 0) {
-        wave_value[wave] = nbh_word_of(acc);
+        wave_value[wave] = acc;
         wave_has[wave] = (int)have;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int w = 1; w < kWaves; ++w)
             if (wave_has[w])
-                nbh_take(acc, have, nbh_value_of(wave_value[w]));
+                nbh_take(acc, have, wave_value[w]);
     }
 }
 
@@ -333,9 +394,15 @@ extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce(const char *
         return;
     }
     if (tid == 0) {
-        const nbh_u64 before = __hip_atomic_exchange(&partials[blockIdx.x], nbh_word_of(acc), __ATOMIC_RELAXED,
-                                                     __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("" ::"v"(before) : "memory");  // wait until the exchange has been carried out
+        const nbh_image img = nbh_image_of(acc);
+        nbh_u64 before[kSlotWords];
+#pragma unroll
+        for (int k = 0; k < kSlotWords; ++k)
+            before[k] = __hip_atomic_exchange(&partials[(long long)blockIdx.x * kSlotWords + k], img.w[k],
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int k = 0; k < kSlotWords; ++k)
+            asm volatile("" ::"v"(before[k]) : "memory");  // wait until the exchanges have been carried out
         const unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last_block = (t == gridDim.x - 1);
         if (last_block)
@@ -345,13 +412,205 @@ extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce(const char *
     if (!last_block)
         return;
     have = false;
-    for (int k = tid; k < (int)gridDim.x; k += kThreads)
-        nbh_take(acc, have, nbh_value_of(__hip_atomic_load(&partials[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)));
+    for (int k = tid; k < (int)gridDim.x; k += kThreads) {
+        nbh_image img;
+#pragma unroll
+        for (int w = 0; w < kSlotWords; ++w)
+            img.w[w] = __hip_atomic_load(&partials[(long long)k * kSlotWords + w], __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+        nbh_take(acc, have, img.value);
+    }
     nbh_fold_workgroup(acc, have);
     if (tid == 0) {
         out[0] = nbh_op(acc, init);
         // leave the scratch buffer as the caller handed it over
         __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// ---- the reference's order of association ---------------------------------------------
+// nbh_custom_reduce_ordered: every application of the operation on the same pair of values,
+// in the same order, as a run of the reference's kernels (kernels/reduction.py:22-166 launched
+// as in :233-258) - for operations that are not associative, or whose rounding depends on the
+// order.  With F = n rounded down to a multiple of 128 and G = min(F / 128, 64) blocks of 128
+// threads, thread g < S = 128 G folds a[g], a[g + S], ... below F from left to right (:70-78);
+// a warp of 32 is the tree (l, l + 16), (l, l + 8) ... (:22-41); a block is (w0 op w2) op
+// (w1 op w3) (:88-97); block 0 takes `init` in (:163-164); the n - F values behind and the
+// partials go through the one-block routine (:99-141, :256-258).
+// One workgroup per warp of the reference: 32 chains whose items lie side by side in every
+// row of S items.  All 512 lanes load rows of 32 items into one of two LDS buffers, a batch
+// at a time, the next batch travelling while lanes 0 - 31 fold the parked one down their
+// chains.  Warp results are published like the partials above; the workgroup that draws the
+// last ticket does the small rest the way the reference's kernels do.
+constexpr int kRefWarp = 32, kRefBlock = 128, kRefMaxGrid = 64;
+constexpr int kOrdRows = (512 / (int)sizeof(T)) > 128 ? 128 : (512 / (int)sizeof(T));  // rows parked per batch
+constexpr int kOrdLoads = kOrdRows * kRefWarp / kThreads;                                // loads per lane and batch
+
+// the reference's one-block routine (:99-141) over m <= 128 values, by one thread: a full warp
+// that is not the last is a tree, the last warp a left fold, and so are the warps
+__device__ T nbh_ref_one_block(const T *v, int m)
+{
+    const int nw = (m + kRefWarp - 1) / kRefWarp;
+    T result = v[0];
+    for (int w = 0; w < nw; ++w) {
+        T wres;
+        if ((w + 1) * kRefWarp < m) {
+            T t[kRefWarp];
+            for (int l = 0; l < kRefWarp; ++l)
+                t[l] = v[w * kRefWarp + l];
+            for (int width = kRefWarp / 2; width; width /= 2)
+                for (int l = 0; l < width; ++l)
+                    t[l] = nbh_op(t[l], t[l + width]);
+            wres = t[0];
+        } else {
+            wres = v[w * kRefWarp];
+            for (int i = 1; i < m - w * kRefWarp; ++i)
+                wres = nbh_op(wres, v[w * kRefWarp + i]);
+        }
+        result = w == 0 ? wres : nbh_op(result, wres);
+    }
+    return result;
+}
+
+extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce_ordered(const char *__restrict__ in, long long n,
+                                                                           long long stride, T init,
+                                                                           T *__restrict__ out,
+                                                                           nbh_u64 *__restrict__ partials,
+                                                                           unsigned *__restrict__ ticket)
+{
+    __shared__ T rows[2][kOrdRows][kRefWarp];
+    __shared__ T small[kRefBlock + 1 + kRefMaxGrid + 1];
+    __shared__ bool last_block;
+    const int tid = threadIdx.x;
+    const long long full = (n / kRefBlock) * kRefBlock;
+    long long ref_grid = full / kRefBlock;
+    if (ref_grid > kRefMaxGrid)
+        ref_grid = kRefMaxGrid;
+    const long long S = ref_grid * kRefBlock;      // chains; 0 when n < 128
+    const int warps = (int)(S / kRefWarp);         // = workgroups with chains
+
+    if ((int)blockIdx.x < warps) {
+        // each XCD (workgroups are dealt to the eight in turn) takes a run of neighbouring
+        // warps: a contiguous piece of every row
+        int warp = (int)blockIdx.x;
+        if (warps % 8 == 0)
+            warp = (warp % 8) * (warps / 8) + warp / 8;
+        const long long c0 = (long long)warp * kRefWarp;
+        const long long nrows = (full - c0 + S - 1) / S;   // items per chain, the same for the 32 of a warp
+        const int chain = tid % kRefWarp, row0 = tid / kRefWarp;
+        constexpr int kRowStep = kThreads / kRefWarp;
+        T held[kOrdLoads];
+        auto fetch = [&](long long first_row) {     // rows behind the last repeat the last: parked, never folded
+#pragma unroll
+            for (int k = 0; k < kOrdLoads; ++k) {
+                long long r = first_row + row0 + k * kRowStep;
+                r = r < nrows ? r : nrows - 1;
+                held[k] = *reinterpret_cast<const T *>(in + (r * S + c0 + chain) * stride);
+            }
+        };
+        T acc = T();
+        const long long nb = (nrows + kOrdRows - 1) / kOrdRows;
+        fetch(0);
+        for (long long b = 0; b < nb; ++b) {
+            const int buf = (int)(b & 1);
+#pragma unroll
+            for (int k = 0; k < kOrdLoads; ++k)
+                rows[buf][row0 + k * kRowStep][chain] = held[k];
+            // one barrier per batch: whoever parks into a buffer next has passed the barrier
+            // that the folding lanes reached after reading it
+            __syncthreads();
+            if (b + 1 < nb)
+                fetch((b + 1) * kOrdRows);
+            if (tid < kRefWarp) {
+                const long long left = nrows - b * kOrdRows;
+                const int count = (int)(left < kOrdRows ? left : kOrdRows);
+                int r = 0;
+                if (b == 0) {                       // a chain starts with its first value
+                    acc = rows[buf][0][tid];
+                    r = 1;
+                }
+                for (; r + 8 <= count; r += 8) {
+                    T v[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        v[j] = rows[buf][r + j][tid];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        acc = nbh_op(acc, v[j]);
+                }
+                for (; r < count; ++r)
+                    acc = nbh_op(acc, rows[buf][r][tid]);
+            }
+        }
+        if (tid < 64) {                             // the first wavefront, whole: the shuffles need its lanes
+#pragma unroll
+            for (int width = kRefWarp / 2; width; width /= 2) {
+                const nbh_image mine = nbh_image_of(acc);
+                nbh_image theirs;
+#pragma unroll
+                for (int w = 0; w < kSlotWords; ++w)
+                    theirs.w[w] = __shfl_down(mine.w[w], width, 64);
+                if (tid < width)
+                    acc = nbh_op(acc, theirs.value);
+            }
+            if (tid == 0) {
+                const nbh_image img = nbh_image_of(acc);
+                nbh_u64 before[kSlotWords];
+#pragma unroll
+                for (int w = 0; w < kSlotWords; ++w)
+                    before[w] = __hip_atomic_exchange(&partials[(long long)warp * kSlotWords + w], img.w[w],
+                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int w = 0; w < kSlotWords; ++w)
+                    asm volatile("" ::"v"(before[w]) : "memory");  // carried out before the ticket is drawn
+            }
+        }
+        __syncthreads();
+    }
+    if (gridDim.x > 1) {
+        if (tid == 0) {
+            const unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_block = (t == gridDim.x - 1);
+            if (last_block)
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        }
+        __syncthreads();
+        if (!last_block)
+            return;
+    }
+
+    // the small rest: small[0 .. 127] the values behind `full`, small[129 ...] one value per block
+    const int m_tail = (int)(n - full);
+    T *tail = small, *part = small + kRefBlock + 1;
+    if (tid < m_tail)
+        tail[tid] = *reinterpret_cast<const T *>(in + (full + tid) * stride);
+    if (tid < (int)ref_grid) {                      // block = (w0 op w2) op (w1 op w3)
+        T w[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            nbh_image img;
+#pragma unroll
+            for (int k = 0; k < kSlotWords; ++k)
+                img.w[k] = __hip_atomic_load(&partials[((long long)tid * 4 + q) * kSlotWords + k], __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+            w[q] = img.value;
+        }
+        part[tid] = nbh_op(nbh_op(w[0], w[2]), nbh_op(w[1], w[3]));
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int np = (int)ref_grid;
+        if (ref_grid)
+            part[0] = nbh_op(part[0], init);
+        if (m_tail) {
+            part[np] = nbh_ref_one_block(tail, m_tail);
+            if (!ref_grid)
+                part[0] = nbh_op(part[0], init);
+            ++np;
+        }
+        out[0] = np > 1 ? nbh_ref_one_block(part, np) : part[0];
+        if (gridDim.x > 1)
+            __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 )NBHSRC";
@@ -363,7 +622,7 @@ struct CustomOp {
     std::mutex lock;
     struct Loaded {
         hipModule_t module = nullptr;
-        hipFunction_t reduce = nullptr;
+        hipFunction_t reduce = nullptr, ordered = nullptr;
     } on_device[kMaxDevices];
 };
 
@@ -387,14 +646,17 @@ int functions_for(CustomOp *op, CustomOp::Loaded **out)
     if (!slot.reduce) {
         hipModule_t m = nullptr;
         NBH_TRY(hipModuleLoadData(&m, op->code.data()));
-        hipFunction_t f = nullptr;
-        const hipError_t e = hipModuleGetFunction(&f, m, "nbh_custom_reduce");
+        hipFunction_t f = nullptr, g = nullptr;
+        hipError_t e = hipModuleGetFunction(&f, m, "nbh_custom_reduce");
+        if (e == hipSuccess)
+            e = hipModuleGetFunction(&g, m, "nbh_custom_reduce_ordered");
         if (e != hipSuccess) {
             (void)hipModuleUnload(m);
             return (int)e;
         }
         slot.module = m;
         slot.reduce = f;
+        slot.ordered = g;
     }
     *out = &slot;
     return 0;
@@ -414,9 +676,9 @@ extern "C" int nbh_reduce_compile(int dtype, const char *body, void **op_out, ch
         put_log(log, log_bytes, "the HIP run-time compiler (libhiprtc.so) could not be loaded");
         return (int)hipErrorSharedObjectInitFailed;
     }
-    std::string source = std::string("typedef ") + type + " T;\n" + kSource;
-    const size_t at = source.find("@BODY@");
-    source.replace(at, 6, body);
+    std::string source = kSource;
+    source.replace(source.find("@T@"), 3, type);
+    source.replace(source.find("@BODY@"), 6, body);
 
     hiprtcProgram prog = nullptr;
     if (r.create(&prog, source.c_str(), "nbh_reduce_custom.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS)
@@ -533,5 +795,35 @@ extern "C" int nbh_reduce_custom(void *handle, const void *in, int64_t n, int64_
     void *args[] = {&in_arg, &n_arg, &head, &units, &stride_arg, &packed_arg, const_cast<void *>(init),
                     &out, &partials, &ticket};
     NBH_TRY(hipModuleLaunchKernel(fn->reduce, (unsigned)grid, 1, 1, kBlock, 1, 1, 0, s, args, nullptr));
+    return 0;
+}
+
+extern "C" int nbh_reduce_custom_ordered(void *handle, const void *in, int64_t n, int64_t in_stride, const void *init,
+                                         void *out, void *scratch, size_t scratch_bytes, nbh_stream_t stream)
+{
+    CustomOp *op = static_cast<CustomOp *>(handle);
+    if (!op || !in || !init || !out || !scratch || n < 1 || scratch_bytes < kNeededBytes ||
+        ((uintptr_t)scratch) % 8 != 0 || in_stride % (int64_t)op->elem != 0)
+        return (int)hipErrorInvalidValue;
+    if (((uintptr_t)in) % op->elem != 0 || ((uintptr_t)out) % op->elem != 0)
+        return (int)hipErrorInvalidValue;
+    CustomOp::Loaded *fn = nullptr;
+    const int rc = functions_for(op, &fn);
+    if (rc)
+        return rc;
+    hipStream_t s = nbh_hip_stream(stream);
+    nbh_stream_report report(s);
+
+    // one workgroup per warp of the reference's launch (at most 64 blocks of four warps)
+    int64_t ref_grid = n / 128;
+    if (ref_grid > 64)
+        ref_grid = 64;
+    const int64_t grid = ref_grid ? ref_grid * 4 : 1;
+    const char *in_arg = static_cast<const char *>(in);
+    long long n_arg = n, stride_arg = in_stride;
+    uint64_t *partials = reinterpret_cast<uint64_t *>(static_cast<char *>(scratch) + kHeaderBytes);
+    unsigned *ticket = reinterpret_cast<unsigned *>(scratch);
+    void *args[] = {&in_arg, &n_arg, &stride_arg, const_cast<void *>(init), &out, &partials, &ticket};
+    NBH_TRY(hipModuleLaunchKernel(fn->ordered, (unsigned)grid, 1, 1, kBlock, 1, 1, 0, s, args, nullptr));
     return 0;
 }

@@ -9,16 +9,27 @@ compiler turns that into kernels (csrc/reduce_custom.hip).
 
 What a functor may do: + - * / // % ** (integer powers: constant exponent), & | ^ << >> ~,
 unary minus, abs(), comparisons, `x if cond else y`, if / else statements, and / or / not
-on conditions, min() / max(), numeric constants (also from globals and closures), and the
-functions of `math` listed in _MATH (also as numpy functions of the same name).  Anything
-else - loops over data, int(), float(), attribute access, calls to other functions with
-side effects - raises NotImplementedError with the reason.
+on conditions, min() / max(), numeric constants (also from globals and closures), the
+functions of `math` listed in _MATH (also as numpy functions of the same name), and
+`.real`, `.imag`, `.conjugate()`.  Anything else - loops over data, int(), float(), other
+attributes, calls to other functions with side effects - raises NotImplementedError with
+the reason.
+
+Complex elements (complex64 / complex128) and complex constants: + - * / and unary minus
+as the JIT lowers them (numba/cuda/cpython/numbers.py:1091-1196: the product is
+(ac - bd) + (ad + bc)i, the quotient CPython's algorithm), == and !=, abs() (hypot),
+z ** 2 (a product, :1062-1078; other powers are not translated), .real / .imag /
+.conjugate() (:1003-1024).  What Python refuses for complex numbers is refused here with
+the same TypeError: ordering comparisons, // and %, bitwise operators, `math` functions.
 
 Typing rules restated from the reference's JIT (numba's integer typing: operations on
 integers are carried out in 64 bits, signed unless both operands are unsigned; a boolean
 in arithmetic is an int64; true division gives float64 for integers; float32 stays
 float32 among float32 operands and becomes float64 with Python floats or integers;
-math.floor / math.ceil return int64; the result is converted to the element type).
+math.floor / math.ceil return int64; complex64 stays complex64 with float32 and complex64
+operands and becomes complex128 with anything wider, Python complex constants are
+complex128; the result is converted to the element type - except complex to real, which the
+JIT refuses too).
 """
 
 import math
@@ -63,6 +74,7 @@ _BINARY = {"add": "__add__", "sub": "__sub__", "mul": "__mul__", "truediv": "__t
            "xor": "__xor__", "lshift": "__lshift__", "rshift": "__rshift__"}
 _COMPARE = {"lt": "__lt__", "le": "__le__", "gt": "__gt__", "ge": "__ge__", "eq": "__eq__", "ne": "__ne__"}
 _UNARY = {"neg": "__neg__", "pos": "__pos__", "abs": "__abs__", "invert": "__invert__"}
+_PARTS = ("real", "imag", "conj")           # .real, .imag, .conjugate(): unary nodes too
 
 # math function -> (C name for double, arity, result): "f" float like the argument,
 # "i" int64 (floor / ceil / trunc), "b" boolean
@@ -94,6 +106,7 @@ _UFUNC_OPERATOR = {
     "greater_equal": ("ge", (0, 1)), "equal": ("eq", (0, 1)), "not_equal": ("ne", (0, 1)),
     "negative": ("neg", (0,)), "positive": ("pos", (0,)), "absolute": ("abs", (0,)), "fabs": ("abs", (0,)),
     "invert": ("invert", (0,)), "bitwise_not": ("invert", (0,)),
+    "conjugate": ("conj", (0,)),
 }
 
 
@@ -102,7 +115,7 @@ def _lift(x):
         return x.expr
     if isinstance(x, (bool, np.bool_)):
         return Expr("const", value=bool(x))
-    if isinstance(x, (int, float, np.integer, np.floating)):
+    if isinstance(x, (int, float, complex, np.integer, np.floating, np.complexfloating)):
         return Expr("const", value=x)
     raise Untranslatable("an operand of type %s is mixed into the computation" % type(x).__name__)
 
@@ -186,6 +199,20 @@ class _Value:
 
     def __round__(self, *_):
         self._refuse("round()")
+
+    def __complex__(self):
+        self._refuse("complex()")
+
+    @property
+    def real(self):
+        return _Value(Expr("real", (self.expr,)), self.script)
+
+    @property
+    def imag(self):
+        return _Value(Expr("imag", (self.expr,)), self.script)
+
+    def conjugate(self):
+        return _Value(Expr("conj", (self.expr,)), self.script)
 
 
 def _install_operators():
@@ -337,10 +364,11 @@ def trace(functor):
 
 _B1, _I64, _U64 = np.dtype(np.bool_), np.dtype(np.int64), np.dtype(np.uint64)
 _F16, _F32, _F64 = np.dtype(np.float16), np.dtype(np.float32), np.dtype(np.float64)
+_C64, _C128 = np.dtype(np.complex64), np.dtype(np.complex128)
 _CTYPE = {np.dtype(np.int8): "signed char", np.dtype(np.int16): "short", np.dtype(np.int32): "int",
           _I64: "nbh_i64", np.dtype(np.uint8): "unsigned char", np.dtype(np.uint16): "unsigned short",
           np.dtype(np.uint32): "unsigned int", _U64: "nbh_u64", _F16: "_Float16", _F32: "float", _F64: "double",
-          _B1: "bool"}
+          _B1: "bool", _C64: "nbh_c64", _C128: "nbh_c128"}
 
 
 def _machine(t):
@@ -352,8 +380,19 @@ def _machine(t):
     return t
 
 
+def _part(t):
+    """Type of the real and imaginary parts of a complex type."""
+    return _F32 if t == _C64 else _F64
+
+
 def _common(t1, t2):
     t1, t2 = _machine(t1), _machine(t2)
+    if t1.kind == "c" or t2.kind == "c":
+        # the complex type whose parts hold both: float32 parts only among complex64,
+        # float32 and float16
+        r1 = _part(t1) if t1.kind == "c" else t1
+        r2 = _part(t2) if t2.kind == "c" else t2
+        return _C64 if _common(r1, r2) in (_F16, _F32) else _C128
     if t1.kind in "iu" and t2.kind in "iu":
         return _U64 if (t1 == _U64 and t2 == _U64) else _I64
     if t1.kind == "f" and t2.kind == "f":
@@ -366,6 +405,14 @@ def _common(t1, t2):
 def _convert(code, src, dst):
     if src == dst:
         return code
+    if src.kind == "c" and dst.kind != "c" and dst != _B1:
+        raise TypeError("cannot convert %s to %s" % (src, dst))          # the JIT has no such cast either
+    if dst.kind == "c":
+        if src == _F16:
+            code = "(float)(%s)" % code
+        return "nbh_cplx_from<%s>(%s)" % (_CTYPE[_part(dst)], code)
+    if dst == _B1 and src.kind == "c":
+        return "((%s) != nbh_cplx_from<%s>(0))" % (code, _CTYPE[_part(src)])
     if dst == _B1:
         return "((%s) != 0)" % code
     if src == _F16 and dst.kind in "iub":
@@ -407,6 +454,8 @@ class _Writer:
             return self.call(e)
         if op in _UNARY:
             return self.unary(op, *self.emit(e.args[0]))
+        if op in _PARTS:
+            return self.part(op, *self.emit(e.args[0]))
         x, tx = self.emit(e.args[0])
         y, ty = self.emit(e.args[1])
         if op in _COMPARE:
@@ -423,6 +472,12 @@ class _Writer:
             return _convert(_float_literal(v), _F64, t), t
         if isinstance(v, float):
             return _float_literal(v), _F64
+        if isinstance(v, (complex, np.complexfloating)):
+            t = np.dtype(type(v)) if isinstance(v, np.complexfloating) else _C128
+            if t not in (_C64, _C128):
+                raise Untranslatable("constant of type %s" % t)
+            r = _CTYPE[_part(t)]
+            return "%s{(%s)%s, (%s)%s}" % (_CTYPE[t], r, _float_literal(v.real), r, _float_literal(v.imag)), t
         if isinstance(v, np.integer):
             t = _machine(np.dtype(type(v)))
             v = int(v)
@@ -436,11 +491,29 @@ class _Writer:
             return "(-9223372036854775807LL - 1LL)", _I64
         return "(%dLL)" % v, _I64
 
+    def part(self, op, x, tx):
+        """.real / .imag / .conjugate(): parts of a complex number; a real number is its own
+        real part and conjugate, its imaginary part a zero of its type
+        (numba/cuda/cpython/numbers.py:1003-1046)."""
+        if tx.kind == "c":
+            if op == "conj":
+                return "nbh_conj(%s)" % x, tx
+            return "(%s).%s" % (x, "re" if op == "real" else "im"), _part(tx)
+        if op == "imag":
+            return _convert("0", _I64, tx), tx
+        return x, tx
+
     def unary(self, op, x, tx):
         t = _machine(tx)
         x = _convert(x, tx, t)
         if op == "pos":
             return x, t
+        if t.kind == "c":
+            if op == "neg":
+                return "(-%s)" % x, t
+            if op == "abs":
+                return "nbh_cabs(%s)" % x, _part(t)
+            raise TypeError("bad operand type for unary ~: %s" % t)
         if t.kind in "iu":
             if op == "neg":
                 return "(%s)(0ULL - (nbh_u64)%s)" % (_CTYPE[t], x), t
@@ -460,6 +533,8 @@ class _Writer:
     def compare(self, op, x, tx, y, ty):
         sign = {"lt": "<", "le": "<=", "gt": ">", "ge": ">=", "eq": "==", "ne": "!="}[op]
         mx, my = _machine(tx), _machine(ty)
+        if (mx.kind == "c" or my.kind == "c") and op not in ("eq", "ne"):
+            raise TypeError("'%s' not supported between %s and %s" % (sign, tx, ty))
         if {mx, my} == {_I64, _U64}:
             # value comparison of a signed with an unsigned number
             if mx == _U64:
@@ -489,6 +564,17 @@ class _Writer:
                 return "(%s)((nbh_u64)%s << %s)" % (_CTYPE[t], _convert(x, tx, t), amount), t
             return "(%s >> %s)" % (_convert(x, tx, t), amount), t
         t = _common(tx, ty)
+        if t.kind == "c":
+            if op == "pow":
+                exponent = e.args[1]
+                if exponent.op != "const" or exponent.value != 2:
+                    raise Untranslatable("complex ** is translated for the exponent 2 only")
+                base = _convert(x, tx, t)
+                return "(%s * %s)" % (base, base), t
+            if op in ("floordiv", "mod"):
+                raise TypeError("can't take floor or mod of complex number")       # Python's words
+            sign = {"add": "+", "sub": "-", "mul": "*", "truediv": "/"}[op]
+            return "(%s %s %s)" % (_convert(x, tx, t), sign, _convert(y, ty, t)), t
         if op == "truediv":
             if t.kind in "iu":
                 t = _F64
@@ -521,6 +607,8 @@ class _Writer:
         args = [self.emit(x) for x in e.args]
         # float32 arguments keep the function in float32; anything else computes in float64
         kinds = [_machine(t) for _, t in args]
+        if any(t.kind == "c" for t in kinds):
+            raise TypeError("can't convert complex to float (math.%s)" % name)      # Python's words
         if all(t in (_F32, _F16) for t in kinds):
             w, cname = _F32, (cname if result == "b" else cname + "f")
         else:

@@ -190,9 +190,10 @@ class Reduce:
         sums and products - and what max / min make of NaN and signed zeros - come out bit for
         bit as the reference computes them (about 5 TB/s instead of 7); False uses this
         library's own order (within 2 n eps sum|x| of it); None takes the setting of
-        NUMBA_CUDA_REDUCE_REFERENCE_ORDER (default 0).  Integer and boolean results are the
-        same either way.  Applies to the operators with kernels of their own, not to
-        translated functors."""
+        NUMBA_CUDA_REDUCE_REFERENCE_ORDER (default 0).  Integer and boolean results of the
+        operators with kernels of their own are the same either way.  A translated functor
+        (any other operation) is applied in the reference's order too: its result then is the
+        reference's also where the operation is not associative."""
         self._functor = functor
         if reference_order is None:
             reference_order = bool(_config.CUDA_REDUCE_REFERENCE_ORDER)
@@ -377,19 +378,22 @@ class Reduce:
         scratch = ctx.reduce_scratch(hstream)
         init_ptr = _init_buffer(dtype, init)
         lib = _driver.driver.lib
+        launch, name = lib.nbh_reduce_custom, "nbh_reduce_custom"
+        if self._ordered:                        # the reference's association: its own entry point
+            launch, name = lib.nbh_reduce_custom_ordered, "nbh_reduce_custom_ordered"
         if res is not None:
             _check_result_array(res, dtype)
-            rc = lib.nbh_reduce_custom(handle, in_ptr, n, arr.strides[0], init_ptr, res.device_ctypes_pointer.value,
-                                       scratch[0], scratch[1], hstream or None)
+            rc = launch(handle, in_ptr, n, arr.strides[0], init_ptr, res.device_ctypes_pointer.value,
+                        scratch[0], scratch[1], hstream or None)
             if rc:
-                _driver.driver.check("nbh_reduce_custom", rc)
+                _driver.driver.check(name, rc)
             return None
         cell = ctx.take_result_cell()
         try:
-            rc = lib.nbh_reduce_custom(handle, in_ptr, n, arr.strides[0], init_ptr, cell[0],
-                                       scratch[0], scratch[1], hstream or None)
+            rc = launch(handle, in_ptr, n, arr.strides[0], init_ptr, cell[0],
+                        scratch[0], scratch[1], hstream or None)
             if rc:
-                _driver.driver.check("nbh_reduce_custom", rc)
+                _driver.driver.check(name, rc)
             _driver.driver.nbh_stream_synchronize(hstream or None)
             return cell[1][:dtype.itemsize].view(dtype)[0]
         finally:
@@ -422,7 +426,7 @@ def compile_translated(expr, dtype):
     import ctypes
     body = _functor.body_for(expr, dtype)
     code = _DTYPE_CODE[np.dtype(np.uint8)] if dtype == _BOOL else _DTYPE_CODE.get(dtype)
-    if code is None or dtype.kind == "c":
+    if code is None:
         raise NotImplementedError("Reduce with a general functor does not support dtype %s" % dtype)
     key = (body, code)
     handle = _COMPILED.get(key)

@@ -192,6 +192,12 @@ def typed_functor(functor, dtype):
                 no intermediate value leaves 64 bits), the result wraps to the type
       booleans  operands are bools, the result is `!= 0`
       float64   Python floats are float64
+      complex128  Python complex numbers: their product is (ac - bd) + (ad + bc)i and their
+                quotient CPython's algorithm, which is what the JIT lowers
+                (numba/cuda/cpython/numbers.py:1123-1179)
+      complex64  NumPy scalars: sums, differences and products part by part in float32
+                like the JIT's; NumPy's QUOTIENT is another algorithm (it multiplies by a
+                reciprocal), so complex64 functors that divide agree to rounding only
       float32 / float16  NumPy scalars of that type.  A Python float constant in the
                 functor makes the JIT compute that step in float64, NumPy keeps it in
                 the narrow type: such functors agree to the narrow type's rounding."""
@@ -213,6 +219,8 @@ def typed_functor(functor, dtype):
         return lambda a, b: np.bool_(bool(functor(bool(a), bool(b))))
     if dtype == np.dtype(np.float64):
         return lambda a, b: np.float64(functor(float(a), float(b)))
+    if dtype == np.dtype(np.complex128):
+        return lambda a, b: np.complex128(functor(complex(a), complex(b)))
     scalar = dtype.type
     narrow = _with_narrow_math(functor, scalar)
 

@@ -14,6 +14,7 @@ SIGNED = ("int8", "int16", "int32", "int64")
 UNSIGNED = ("uint8", "uint16", "uint32", "uint64")
 INTS = SIGNED + UNSIGNED
 FLOATS = ("float32", "float64")
+COMPLEX = ("complex64", "complex128")
 
 _weight = 3          # read from the module's globals by a functor below
 
@@ -57,6 +58,8 @@ class Case:
         low, high = self.low, self.high
         if dtype == np.float16:
             low, high = max(low, -60000), min(high, 60000)
+        if dtype.kind == "c":
+            return ((rng.random(n) * (high - low) + low) + 1j * (rng.random(n) * (high - low) + low)).astype(dtype)
         return (rng.random(n) * (high - low) + low).astype(dtype)
 
     def __repr__(self):
@@ -102,6 +105,17 @@ CASES = [
     Case("float_constant", lambda a, b: 0.5 * a + b, FLOATS + ("int32",), -10**4, 10**4, exact=False),
     Case("nan_aware", lambda a, b: b if math.isnan(a) else a, FLOATS, -1, 1),
     Case("tangent", lambda a, b: math.atan2(a, b) + math.tanh(a), FLOATS, -3, 3, exact=False),
+    # complex elements (complex64 only where nothing divides: see oracle.cref.typed_functor)
+    Case("complex_sum_plus_i", lambda a, b: a + b + 1j, COMPLEX, -100, 100, fold=True, init=2 - 1j),
+    Case("complex_product_mix", lambda a, b: a * b + a - b, COMPLEX, -2, 2),
+    Case("complex_quotient", lambda a, b: a / (b + 2) - b / a, ("complex128",), -1.5, 1.5),
+    Case("complex_quotient_narrow", lambda a, b: a / (b + 2), ("complex64",), -1.5, 1.5, exact=False),
+    Case("conjugate_and_parts", lambda a, b: a.conjugate() * b + (a.real - b.imag), COMPLEX, -2, 2),
+    Case("parts_of_real_numbers", lambda a, b: a.real + b.conjugate() - a.imag, ("int32", "float64"), -1000, 1000),
+    Case("square_and_compare", lambda a, b: a ** 2 if a != b else -b, ("complex128",), -2, 2),
+    Case("modulus", lambda a, b: abs(a) + abs(b) * 1j, COMPLEX, -3, 3, exact=False),
+    Case("truth_of_complex", lambda a, b: a if a and not b == 0 else b + (1 + 2j), COMPLEX, -1, 1),
+    Case("numpy_complex_constant", lambda a, b: np.complex64(0.5 + 0.25j) * np.conjugate(b) + a, COMPLEX, -8, 8),
 ]
 
 BY_NAME = {c.name: c for c in CASES}
@@ -116,4 +130,17 @@ REFUSED = [
     (lambda a, b: a[0] + b, "indexing"),
     (lambda a, b: a + "x", "TypeError"),
     (lambda a, b: np.cumsum(a), "not a number"),
+    (lambda a, b: complex(a) + b, "complex()"),
+    (lambda a, b: a.bit_length() + b, "AttributeError"),
+]
+
+# refused for complex elements with Python's own TypeError, when the element type is known
+COMPLEX_TYPE_ERRORS = [
+    (lambda a, b: a if a > b else b, "not supported"),
+    (lambda a, b: max(a, b), "not supported"),
+    (lambda a, b: a // b, "floor"),
+    (lambda a, b: a % b, "floor or mod"),
+    (lambda a, b: a ^ b, "bitwise"),
+    (lambda a, b: math.sqrt(a) + b, "complex to float"),
+    (lambda a, b: ~a + b, "unary"),
 ]

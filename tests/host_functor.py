@@ -16,21 +16,24 @@ _SRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "numba_cud
 
 CTYPE = {"int8": "signed char", "int16": "short", "int32": "int", "int64": "long long",
          "uint8": "unsigned char", "uint16": "unsigned short", "uint32": "unsigned int",
-         "uint64": "unsigned long long", "float32": "float", "float64": "double", "bool": "unsigned char"}
+         "uint64": "unsigned long long", "float32": "float", "float64": "double", "bool": "unsigned char",
+         "complex64": "nbh_c64", "complex128": "nbh_c128"}
 
 
-def helpers():
+def helpers(ctype):
+    """The device source up to nbh_op, with the element type put in where the library puts it."""
     text = open(_SRC).read()
     start = text.index('R"NBHSRC(') + len('R"NBHSRC(')
     stop = text.index("__device__ __forceinline__ T nbh_op(T a, T b)")
     part = text[start:stop]
-    return re.sub(r"typedef unsigned int nbh_u32x4[^\n]*\n", "", part)
+    assert part.count("@T@") == 1
+    return re.sub(r"typedef unsigned int nbh_u32x4[^\n]*\n", "", part).replace("@T@", ctype)
 
 
 def build(bodies, dtype_name):
     """-> list of callables f(a, b) -> array, one per body, for arrays of the dtype."""
     src = ["#include <cmath>", "#include <cstdint>", "using namespace std;", "#define __device__",
-           "#define __forceinline__ inline", "typedef %s T;" % CTYPE[dtype_name], helpers()]
+           "#define __forceinline__ inline", helpers(CTYPE[dtype_name])]
     for k, body in enumerate(bodies):
         src.append("static inline T op_%d(T a, T b)\n{\n%s\n}" % (k, body))
         src.append('extern "C" void apply_%d(const T *a, const T *b, T *out, long n)\n'

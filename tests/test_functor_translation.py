@@ -24,7 +24,8 @@ from oracle import cref
 from tests import functor_cases as FC
 from tests import host_functor
 
-DTYPES = ["int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64", "float32", "float64", "bool"]
+DTYPES = ["int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64", "float32", "float64", "bool",
+          "complex64", "complex128"]
 
 
 def _ulps(got, want):
@@ -50,8 +51,16 @@ def test_translated_bodies_agree_with_the_functor(dtype_name):
         got = apply(a, b)
         # float32 elements with Python constants: the JIT (and the body) take that step in
         # float64, the oracle's NumPy scalars stay in float32
-        widened = dtype == np.float32 and "(double)" in body
-        if dtype.kind != "f" or (case.exact and not widened):
+        widened = (dtype == np.float32 and "(double)" in body) or (dtype == np.complex64 and "<double>" in body)
+        if dtype.kind == "c" and not (case.exact and not widened):
+            # complex: the same 4 units, of the larger part (hypot and the quotient differ by a unit or two)
+            part = np.float32 if dtype == np.complex64 else np.float64
+            scale = np.maximum(np.abs(want.real), np.abs(want.imag)).astype(np.float64)
+            if widened:
+                scale = scale + 8 * (np.abs(a) + np.abs(b)).astype(np.float64)
+            err = np.maximum(np.abs(got.real.astype(np.float64) - want.real), np.abs(got.imag.astype(np.float64) - want.imag))
+            assert (err / np.spacing(scale.astype(part))).max() <= 4.0, (case, dtype_name)       # tolerance: 4 ulp
+        elif dtype.kind != "f" or (case.exact and not widened):
             bad = np.flatnonzero(got.view(np.uint8).reshape(len(got), -1) != want.view(np.uint8).reshape(len(want), -1))
             assert got.tobytes() == want.tobytes(), (case, dtype_name, a[bad[:3] // dtype.itemsize],
                                                      b[bad[:3] // dtype.itemsize], got[bad[:3] // dtype.itemsize],
@@ -104,8 +113,22 @@ def test_typing_rules_written_as_casts():
     assert F.body_for(e, np.uint32).strip().startswith("return (unsigned int)((nbh_i64)(")
     with pytest.raises(TypeError, match="bitwise"):
         F.body_for(F.trace(lambda a, b: a ^ b ^ 1), np.float32)
-    with pytest.raises(NotImplementedError, match="dtype"):
-        F.body_for(e, np.complex64)
+    # complex: float32 parts only among complex64 and float32 operands; conversions are calls
+    assert F.body_for(F.trace(lambda a, b: a * b + a), np.complex64).strip() == "return ((a * b) + a);"
+    assert "nbh_cplx_from<double>" in F.body_for(e, np.complex64)          # + int64 constant -> complex128
+    assert "nbh_cplx_from<double>" not in F.body_for(F.trace(lambda a, b: a * np.float32(2) + b.real), np.complex64)
+    assert F.body_for(F.trace(lambda a, b: abs(a) + abs(b)), np.complex128).strip() == \
+        "return nbh_cplx_from<double>((nbh_cabs(a) + nbh_cabs(b)));"
+    with pytest.raises(TypeError, match="cannot convert complex"):
+        F.body_for(F.trace(lambda a, b: a + b * 1j), np.float64)        # a complex result for real elements
+
+
+@pytest.mark.parametrize("functor,why", FC.COMPLEX_TYPE_ERRORS)
+def test_what_python_refuses_for_complex_numbers_is_a_type_error(functor, why):
+    tree = F.trace(functor)                      # the trace does not know the element type yet
+    for dtype in (np.complex64, np.complex128):
+        with pytest.raises(TypeError, match=why):
+            F.body_for(tree, dtype)
 
 
 @pytest.mark.parametrize("functor,why", FC.REFUSED)
@@ -146,4 +169,4 @@ def test_every_body_passes_the_run_time_compiler():
     # a body that is not C++ comes back with the compiler's message
     rc = lib.nbh_reduce_compile(2, b"return a +* b;", ctypes.byref(handle), log, len(log))
     assert rc == 300 and b"error" in log.value
-    assert lib.nbh_reduce_compile(10, b"return a;", ctypes.byref(handle), log, len(log)) == 1     # complex: refused
+    assert lib.nbh_reduce_compile(99, b"return a;", ctypes.byref(handle), log, len(log)) == 1     # no such element type

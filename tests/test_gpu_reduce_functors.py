@@ -35,13 +35,15 @@ def _say(*a):
 def _check(case, dtype, got, want, n, data):
     dtype = np.dtype(dtype)
     assert isinstance(got, dtype.type), (case, dtype, type(got))
-    if dtype.kind != "f" or case.selects:
+    if dtype.kind not in "fc" or case.selects:
         assert got.tobytes() == want.tobytes(), (case, dtype, n, got, want)
     else:
         # sums: against the sum of magnitudes; the other folds: against the result
         eps = np.finfo(dtype).eps
-        scale = float(np.abs(data.astype(np.float64)).sum()) + n if case.name == "sum_plus_one" else abs(float(want))
-        assert abs(float(got) - float(want)) <= 4 * max(n, 8) * eps * scale, (case, dtype, n, got, want)
+        wide = np.complex128 if dtype.kind == "c" else np.float64
+        sums = case.name in ("sum_plus_one", "complex_sum_plus_i")
+        scale = float(np.abs(data.astype(wide)).sum()) + n if sums else abs(wide(want))
+        assert abs(wide(got) - wide(want)) <= 4 * max(n, 8) * eps * scale, (case, dtype, n, got, want)
 
 
 @pytest.mark.parametrize("case", FOLDS, ids=repr)
@@ -235,8 +237,10 @@ def test_untranslatable_functor_is_refused_when_the_object_is_made():
         cuda.Reduce(lambda a, b: int(a) + b)
     with pytest.raises(TypeError, match="bitwise"):
         cuda.Reduce(FC.BY_NAME["xor_and_flip"].functor)(np.zeros(4, np.float32))
-    with pytest.raises(NotImplementedError, match="dtype"):
-        cuda.Reduce(FC.BY_NAME["sum_plus_one"].functor)(np.zeros(4, np.complex64))
+    with pytest.raises(TypeError, match="not supported"):          # complex numbers are not ordered
+        cuda.Reduce(FC.BY_NAME["saturating_sum"].functor)(np.zeros(4, np.complex64))
+    with pytest.raises(TypeError, match="cannot convert complex"):  # a complex result for real elements
+        cuda.Reduce(lambda a, b: a + b * 1j)(np.zeros(4, np.float64))
 
 
 def test_max_min_spelled_with_other_comparisons_keep_their_own_nan_rule():
@@ -266,3 +270,109 @@ def test_max_min_spelled_with_other_comparisons_keep_their_own_nan_rule():
         # integers: the native kernels, exact
         ints = rng.integers(-1000, 1000, 5000).astype(np.int32)
         assert red(ints, init=0) == cref.functor_tree(functor, ints, 0)
+
+
+# ---- translated functors in the reference's order of association ---------------------------
+# With reference_order=True every application is made on the same pair of values as in a run
+# of the reference's kernels, so the comparison with oracle.cref.functor_tree is bit for bit
+# also for functors that are NOT associative (a - b, a / 2 + b / 4 ...) and for floating-point
+# roundings that depend on the order.  float32 only with functors whose constants (if any) do
+# not change the precision of a step: a Python number in the functor makes the JIT compute
+# that step in float64 where NumPy scalars, which the oracle runs on, stay in float32
+# (`a + b + 1` is safe: rounding the exact float64 sum once more to float32 gives the float32 sum).
+FLOAT32_SAFE = ("sum_plus_one", "difference", "abs_difference_statement", "spread", "nested_conditions",
+                "largest_magnitude", "nan_aware")
+ORDER_SIZES = [1, 2, 31, 32, 33, 127, 128, 129, 255, 256, 1000, 4099, 8191, 8192, 8192 * 2 + 128 * 5 + 3, 30011]
+
+
+def _ordered_cases():
+    for case in FC.CASES:
+        if not case.exact:
+            continue
+        ints = [d for d in case.dtypes if np.dtype(d).kind in "iu"]
+        chosen = ints[:1] + ints[-1:] if len(ints) > 1 else ints
+        if "float64" in case.dtypes:
+            chosen.append("float64")
+        if "float32" in case.dtypes and case.name in FLOAT32_SAFE:
+            chosen.append("float32")
+        if "bool" in case.dtypes:
+            chosen.append("bool")
+        chosen += [d for d in case.dtypes if d.startswith("complex")]
+        for dtype in chosen:
+            yield pytest.param(case, dtype, id="%s-%s" % (case.name, dtype))
+
+
+def _same_bits(got, want):
+    return got.tobytes() == want.tobytes() or (got != got and want != want)
+
+
+@pytest.mark.parametrize("case,dtype", list(_ordered_cases()))
+def test_translated_functors_in_the_reference_order(case, dtype):
+    red = cuda.Reduce(case.functor, reference_order=True)
+    for n in ORDER_SIZES:
+        _say("ordered", case, dtype, n)
+        data = case.operands(dtype, n, n + 1)
+        want = cref.functor_tree(case.functor, data, case.init)
+        got = red(data, init=case.init)
+        assert isinstance(got, np.dtype(dtype).type)
+        assert _same_bits(got, want), (case, dtype, n, got, want)
+
+
+@pytest.mark.parametrize("name,dtype,n", [("difference", "float32", 8192 * 300 + 12345),
+                                          ("difference", "int16", 8192 * 261 + 77),
+                                          ("sum_plus_one", "float64", 8192 * 150 + 128 * 37),
+                                          ("halves", "float64", 128 * 40 * 70 + 5)])
+def test_reference_order_over_many_batches_of_rows(name, dtype, n):
+    """Chains longer than the rows a workgroup parks at a time (128 rows of 1 - 4 byte items, 64
+    of 8-byte ones), grids below the reference's 64 blocks, views and `res=`."""
+    case = FC.BY_NAME[name]
+    _say("ordered, long", name, dtype, n)
+    data = case.operands(dtype, n, 5)
+    want = cref.functor_tree(case.functor, data, 3)
+    red = cuda.Reduce(case.functor, reference_order=True)
+    d = cuda.to_device(data)
+    assert _same_bits(red(d, init=3), want)
+    res = cuda.device_array(2, dtype)
+    s = cuda.stream()
+    assert red(d, res=res[1:], init=3, stream=s) is None
+    s.synchronize()
+    assert _same_bits(res.copy_to_host()[1], want)
+    every_third = data[::3]
+    assert _same_bits(red(d[::3], init=3), cref.functor_tree(case.functor, every_third, 3))
+    backwards = data[100000:50:-1]
+    assert _same_bits(red(d[100000:50:-1], init=3), cref.functor_tree(case.functor, backwards, 3))
+
+
+def test_reference_order_interleaves_with_the_other_kernels_on_one_scratch_buffer():
+    rng = np.random.default_rng(9)
+    data = rng.standard_normal(200003).astype(np.float32)
+    d = cuda.to_device(data)
+    minus = lambda a, b: a - b
+    ordered = cuda.Reduce(minus, reference_order=True)
+    plain = cuda.Reduce(lambda a, b: a + b + 1)
+    native = cuda.Reduce(lambda a, b: a + b, reference_order=True)
+    want_minus = cref.functor_tree(minus, data, 0.5)
+    want_native = cref.tree("add", data, 0.5)
+    ints = cuda.to_device(np.arange(100000, dtype=np.int64))
+    for _ in range(4):
+        assert _same_bits(ordered(d, init=0.5), want_minus)
+        assert plain(ints) == 99999 * 100000 // 2 + 100000
+        assert _same_bits(native(d, init=0.5), np.float32(want_native))
+
+
+@pytest.mark.parametrize("name", ["modulus", "complex_quotient_narrow"])
+def test_complex_functors_that_call_the_library_or_divide_in_float32(name):
+    """abs() is hypot from the device library, and NumPy, which the oracle runs complex64 on,
+    divides by another algorithm than the JIT: a unit or two in the last place per
+    application.  Reference order, compared part by part within 16 n eps of the larger part."""
+    case = FC.BY_NAME[name]
+    red = cuda.Reduce(case.functor, reference_order=True)
+    for dtype in case.dtypes:
+        eps = np.finfo(dtype).eps
+        for n in (1, 2, 33, 128, 1000, 4099):
+            _say(name, dtype, n)
+            data = case.operands(dtype, n, n)
+            want = cref.functor_tree(case.functor, data, 0.25 + 0.5j)
+            got = red(data, init=0.25 + 0.5j)
+            assert isinstance(got, np.dtype(dtype).type)
+            assert abs(np.complex128(got) - np.complex128(want)) <= 16 * max(n, 8) * eps * abs(np.complex128(want))

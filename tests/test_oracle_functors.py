@@ -55,3 +55,41 @@ def test_typing_of_booleans_and_float_results():
     assert g(np.int32(-3), np.int32(0)) == -1 and isinstance(g(1, 1), np.int32)       # towards zero
     h = cref.typed_functor(lambda a, b: a * b, np.float32)
     assert h(np.float32(1.1), np.float32(1.1)) == np.float32(1.1) * np.float32(1.1)
+
+
+@pytest.mark.parametrize("n", [1, 2, 33, 127, 129, 1000, 8192 + 77, 20000])
+def test_complex_elements_match_the_c_restatement(n):
+    """complex128 runs on Python complex numbers, complex64 on NumPy scalars: sums and products
+    must come out as the C restatement's (part by part; (ac - bd) + (ad + bc)i), in tree and
+    fold order."""
+    rng = np.random.default_rng(n)
+    for dtype in (np.complex64, np.complex128):
+        z = (rng.standard_normal(n) + 1j * rng.standard_normal(n)).astype(dtype)
+        near_one = (1 + z / 64).astype(dtype)
+        for name, functor, data in (("add", lambda a, b: a + b, z), ("mul", lambda a, b: a * b, near_one)):
+            assert cref.functor_tree(functor, data, 0.5 - 2j).tobytes() == cref.tree(name, data, 0.5 - 2j).tobytes()
+            assert cref.functor_fold(functor, data, 0.5 - 2j).tobytes() == cref.fold(name, data, 0.5 - 2j).tobytes()
+
+
+def test_complex128_quotient_is_the_algorithm_the_jit_lowers():
+    """typed_functor divides complex128 with Python's own `/`.  The reference lowers the quotient
+    as written at numba/cuda/cpython/numbers.py:1150-1177 (scale by the larger part of the
+    divisor): Python's must be that algorithm to the bit, also where the two parts of the
+    divisor are equal in size, of opposite sign, or one of them zero."""
+    def lowered(a, b):
+        if abs(b.real) >= abs(b.imag):
+            ratio = b.imag / b.real
+            denom = b.real + b.imag * ratio
+            return complex((a.real + a.imag * ratio) / denom, (a.imag - a.real * ratio) / denom)
+        ratio = b.real / b.imag
+        denom = b.real * ratio + b.imag
+        return complex((a.real * ratio + a.imag) / denom, (a.imag * ratio - a.real) / denom)
+
+    rng = np.random.default_rng(11)
+    a = rng.standard_normal(20000) + 1j * rng.standard_normal(20000)
+    b = rng.standard_normal(20000) * 10.0 ** rng.integers(-3, 4, 20000) + 1j * rng.standard_normal(20000)
+    b[:4] = [1 + 1j, 2 - 2j, 3 + 0j, 0 - 5j]
+    f = cref.typed_functor(lambda x, y: x / y, np.complex128)
+    for x, y in zip(a, b):
+        want = lowered(complex(x), complex(y))
+        assert f(x, y).tobytes() == np.complex128(want).tobytes(), (x, y)
