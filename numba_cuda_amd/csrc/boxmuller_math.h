@@ -31,6 +31,20 @@
 
 namespace bm {
 
+// a * b + c in one instruction whose addend may be a constant in a scalar register.  Left to
+// itself the compiler keeps some addends of a Horner chain in vector registers and copies
+// them before every accumulating multiply-add: one more vector instruction per step.
+BM_FN double fma_const(double a, double b, double c)
+{
+#ifdef __HIP_DEVICE_COMPILE__
+    double d;
+    asm("v_fma_f64 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "s"(c));
+    return d;
+#else
+    return __builtin_fma(a, b, c);
+#endif
+}
+
 // ---- logarithm -------------------------------------------------------------------
 // u = 2^e * m with m in [sqrt(1/2), sqrt(2)).  The 2^23 mantissa patterns of m are cut
 // into 128 runs of 2^16; run j has a centre c_j (1.0 for the run that contains 1.0)
@@ -85,7 +99,10 @@ inline void build_log_table(LogTable &t)
     }
 }
 
-BM_FN double log_positive_f32(float u, const LogTable *__restrict__ tab)
+// `Tab` in the functions below: a pointer to a LogTable - `const LogTable *`, or on the device
+// one that carries the LDS address space, so that the look-ups are LDS instructions with
+// 32-bit addresses.
+template <typename Tab> BM_FN double log_positive_f32(float u, Tab tab)
 {
     uint32_t bits;
 #ifdef __HIP_DEVICE_COMPILE__
@@ -107,9 +124,9 @@ BM_FN double log_positive_f32(float u, const LogTable *__restrict__ tab)
     // r = RN(m * q_j - 1): one rounding, relative to r itself
     const double r = __builtin_fma(m, tab->q[j], -1.0);
     // log1p(r) - r, |r| <= 2^-8: the r^7 / 7 term is below 2^-58
-    double p = __builtin_fma(r, -1.0 / 6.0, 1.0 / 5.0);
-    p = __builtin_fma(r, p, -1.0 / 4.0);
-    p = __builtin_fma(r, p, 1.0 / 3.0);
+    double p = fma_const(r, -1.0 / 6.0, 1.0 / 5.0);
+    p = fma_const(r, p, -1.0 / 4.0);
+    p = fma_const(r, p, 1.0 / 3.0);
     p = __builtin_fma(r, p, -0.5);
     p = (r * r) * p;
     const double ln2_hi = 0x1.62e42feep-1;             // 32 bits of ln 2
@@ -119,7 +136,7 @@ BM_FN double log_positive_f32(float u, const LogTable *__restrict__ tab)
     return hi + (r + lo);                              // the small terms first
 }
 
-BM_FN double bm_log_f32(float u, const LogTable *__restrict__ tab)
+template <typename Tab> BM_FN double bm_log_f32(float u, Tab tab)
 {
     const double v = log_positive_f32(u, tab);
     return (u == 0.0f) ? -HUGE_VAL : v;
@@ -137,7 +154,7 @@ BM_FN double bm_log_f32(float u, const LogTable *__restrict__ tab)
 // instructions are what bounds the generators, so ONE Horner chain runs: the quadrant
 // picks factor, tail and base per lane (32-bit selects) and the row of the coefficient
 // table (loads from LDS on the device, which cost the vector ALU nothing).
-BM_FN double bm_cos_2pi(double x, const LogTable *__restrict__ tab)
+template <typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
 {
     const double inv_pio2 = 0x1.45f306dc9c883p-1;
     const double pio2_1 = 0x1.921fb544p+0;             // first 33 bits of pi/2
@@ -153,7 +170,12 @@ BM_FN double bm_cos_2pi(double x, const LogTable *__restrict__ tab)
     const double y1 = (r - y0) - w2;
 
     const bool odd = (n & 1) != 0;                     // odd quadrant: -+sin, even: +-cos
-    const double *__restrict__ k = tab->trig[n & 1];   // S6..S1 : C6..C1
+    auto k = &tab->trig[n & 1][0];                     // S6..S1 : C6..C1
+#ifdef __HIP_DEVICE_COMPILE__
+    // the row's address as ONE value: the six loads then differ in their offset fields only
+    // (otherwise the compiler hoists "table + 16" and "table + 32" and adds the row to each)
+    asm("" : "+v"(k));
+#endif
     const double z = y0 * y0;
     const double hz = 0.5 * z;
     const double wc = 1.0 - hz;
@@ -169,7 +191,15 @@ BM_FN double bm_cos_2pi(double x, const LogTable *__restrict__ tab)
     const double base = odd ? y0 : wc;
     const double pick = base + __builtin_fma(factor, q, tail);
     // cos(n*pi/2 + y): n&3 = 0: cos y, 1: -sin y, 2: -cos y, 3: sin y
+#ifdef __HIP_DEVICE_COMPILE__
+    // bit 1 of n + 1 moved onto the sign bit and xor-ed in: a shift-and-add and one
+    // three-input bit operation, hi ^ (sign & 0x80000000)
+    const uint32_t sign = ((uint32_t)n << 30) + 0x40000000u;
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_bitop3_b32(__double2hiint(pick), sign, 0x80000000u, 0x78);
+    return __hiloint2double((int)hi, __double2loint(pick));
+#else
     return (((n + 1) & 2) != 0) ? -pick : pick;
+#endif
 }
 
 // Square root of -2 log(u): zero, +infinity or a double in [2^-22, 210] - never

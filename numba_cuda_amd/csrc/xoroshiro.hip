@@ -465,18 +465,22 @@ __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t 
 // carry the two halves in their mantissas; (first - (2^31 + 2^-1)) + second is
 // m * 2^-53, and both additions are exact (every intermediate is a multiple of
 // 2^-53 below 1 in magnitude).
+// The two halves of m are made by two 32-bit instructions, each writing the low word of its
+// double directly (one 64-bit shift would leave them in a register pair, to be moved apart).
 __device__ __forceinline__ double unit_double(uint64_t x)
 {
-    const uint64_t m = shr64<11>(x);
-    const double a = __builtin_bit_cast(double, (uint64_t)0x41E0000000000000ull | (m >> 32));
-    const double b = __builtin_bit_cast(double, (uint64_t)0x3FE0000000000000ull | (m & 0xFFFFFFFFull));
+    const uint32_t x_lo = (uint32_t)x, x_hi = (uint32_t)(x >> 32);
+    const uint32_t m_hi = x_hi >> 11, m_lo = funnel(x_hi, x_lo, 11);
+    const double a = __hiloint2double((int)0x41E00000, (int)m_hi);
+    const double b = __hiloint2double((int)0x3FE00000, (int)m_lo);
     return (a - 2147483648.5) + b;
 }
 
 struct UniformF32 {
     using value_type = float;
     static constexpr bool kHeavy = false;
-    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1, const bm::LogTable * = nullptr)
+    template <typename Tab = const bm::LogTable *>
+    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1, Tab = Tab())
     {
         // the exact value in double, then one rounding to float
         return (float)unit_double(next_d(s0, s1));
@@ -485,7 +489,8 @@ struct UniformF32 {
 struct UniformF64 {
     using value_type = double;
     static constexpr bool kHeavy = false;
-    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1, const bm::LogTable * = nullptr)
+    template <typename Tab = const bm::LogTable *>
+    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1, Tab = Tab())
     {
         return unit_double(next_d(s0, s1));
     }
@@ -496,7 +501,7 @@ struct UniformF64 {
 struct NormalF32 {
     using value_type = float;
     static constexpr bool kHeavy = true;
-    static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1, const bm::LogTable *tab)
+    template <typename Tab> static __device__ __forceinline__ float draw(uint64_t &s0, uint64_t &s1, Tab tab)
     {
         const float u1 = UniformF32::draw(s0, s1);
         const float u2 = UniformF32::draw(s0, s1);
@@ -512,7 +517,7 @@ struct NormalF32 {
 struct NormalF64 {
     using value_type = double;
     static constexpr bool kHeavy = true;
-    static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1, const bm::LogTable *tab)
+    template <typename Tab> static __device__ __forceinline__ double draw(uint64_t &s0, uint64_t &s1, Tab tab)
     {
         const float u1 = UniformF32::draw(s0, s1);
         const float u2 = UniformF32::draw(s0, s1);
@@ -559,7 +564,9 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
 
     // the normal generators look their logarithm up in a 3 KiB table: into LDS first
     __shared__ typename std::conditional<Gen::kHeavy, bm::LogTable, char>::type tab_store;
-    const bm::LogTable *tab = reinterpret_cast<const bm::LogTable *>(&tab_store);
+    // typed as an LDS pointer: the table look-ups are then LDS instructions with 32-bit addresses
+    typedef const __attribute__((address_space(3))) bm::LogTable *LdsTable;
+    const LdsTable tab = (LdsTable)reinterpret_cast<const bm::LogTable *>(&tab_store);
     if (Gen::kHeavy) {
         const double *src = reinterpret_cast<const double *>(log_table);
         double *dst = reinterpret_cast<double *>(&tab_store);
@@ -602,7 +609,7 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
                     } mine;
 #pragma unroll
                     for (int j = 0; j < CHUNK; ++j)
-                        mine.val[j] = Gen::draw(s0, s1, nullptr);
+                        mine.val[j] = Gen::draw(s0, s1, (const bm::LogTable *)nullptr);
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
                         *reinterpret_cast<u32x4 *>(&park[lane][h * CHUNK + k * PER]) = mine.pk[k];
@@ -736,7 +743,7 @@ __global__ __launch_bounds__(kFillBlock) void fill_regs_kernel(uint64_t *__restr
         } mine;
 #pragma unroll
         for (int j = 0; j < ROUND; ++j)
-            mine.val[j] = Gen::draw(s0, s1, nullptr);
+            mine.val[j] = Gen::draw(s0, s1, (const bm::LogTable *)nullptr);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             if (quarter == q) {
@@ -844,7 +851,7 @@ __global__ __launch_bounds__(kFillBlock) void fill_ring_kernel(uint64_t *__restr
                     } mine;
 #pragma unroll
                     for (int j = 0; j < ROUND; ++j)
-                        mine.val[j] = Gen::draw(s0, s1, nullptr);
+                        mine.val[j] = Gen::draw(s0, s1, (const bm::LogTable *)nullptr);
                     // every skew of the launch is a multiple of `grain` values: park in
                     // pieces of that size (they neither straddle the wrap nor lose alignment)
                     if (grain >= PER) {
@@ -875,14 +882,14 @@ __global__ __launch_bounds__(kFillBlock) void fill_ring_kernel(uint64_t *__restr
                     VT four[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        four[e] = Gen::draw(s0, s1, nullptr);
+                        four[e] = Gen::draw(s0, s1, (const bm::LogTable *)nullptr);
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         ring[lane][(col0 + j + e) & (RING - 1)] = four[e];
                 }
 #pragma unroll 1
                 for (; j < m; ++j)
-                    ring[lane][(col0 + j) & (RING - 1)] = Gen::draw(s0, s1, nullptr);
+                    ring[lane][(col0 + j) & (RING - 1)] = Gen::draw(s0, s1, (const bm::LogTable *)nullptr);
             }
             if (r == gen_rounds - 1 && live && lane > 0 && my_skew > 0) {
                 // the run before this one ends `my_skew` values into its last line: the
