@@ -342,23 +342,42 @@ constexpr int64_t kTablesFrom = 1 << 18;  // below this the table load outweighs
 // the 16 rounds every lane visits every position, and in any one round the 16 lanes of a row
 // of the wavefront read 16 different positions - 16 different groups of banks, whatever the
 // values.  Which byte of the state a lane needs in round t then depends on the lane; the state
-// is permuted once per step (bytes by a per-lane v_perm selector, words by conditional swaps) so
-// that round t finds its byte in a fixed place.
+// is permuted once per step so that round t finds its byte in a fixed place: byte i of word j
+// of the permuted state is byte i ^ (l & 3) of word j ^ ((l >> 2) & 3) of the state - the words
+// 0 <-> 2, 1 <-> 3 by conditional moves, the rest by one two-source v_perm_b32 per word.
+// The address of round t is (value << 8) | ((t ^ l) << 4): the low byte never changes, so each
+// round keeps its address register and a step only moves the value into byte 1 of it
+// (one sub-dword move per look-up instead of an extraction and a merge).
 struct LaneOrder {
-    uint32_t byte_select;  // v_perm selector: byte i of the result is byte i ^ (l & 3) of the source
-    bool swap1, swap2;     // exchange words 0<->1, 2<->3 / 0<->2, 1<->3 of the 128-bit state
-    uint32_t base;         // (l mod 16) * 16: this lane's position in round 0, as a byte offset in a table row
+    uint32_t select;   // v_perm selector for (other word, this word): byte and word exchange in one
+    bool swap2;        // exchange words 0 <-> 2, 1 <-> 3 of the 128-bit state
+    uint32_t at[16];   // address of round t within the table: byte 0 = (t ^ l16) << 4, byte 1 = the value
 };
 
 __device__ __forceinline__ LaneOrder lane_order(int lane)
 {
     const uint32_t l16 = (uint32_t)lane & 15u;
     LaneOrder o;
-    o.byte_select = 0x03020100u ^ ((l16 & 3u) * 0x01010101u);
-    o.swap1 = (l16 & 4u) != 0;
+    // selector bytes 0 - 3 pick from the second source, 4 - 7 from the first
+    o.select = (0x03020100u ^ ((l16 & 3u) * 0x01010101u)) | ((l16 & 4u) ? 0x04040404u : 0u);
     o.swap2 = (l16 & 8u) != 0;
-    o.base = l16 << 4;
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+        o.at[t] = (l16 << 4) ^ (uint32_t)(t << 4);
     return o;
+}
+
+// byte K of `w` into byte 1 of `at`, the other bytes of `at` kept
+template <int K> __device__ __forceinline__ void put_row(uint32_t &at, uint32_t w)
+{
+    if constexpr (K == 0)
+        asm("v_mov_b32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0" : "+v"(at) : "v"(w));
+    else if constexpr (K == 1)
+        asm("v_mov_b32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1" : "+v"(at) : "v"(w));
+    else if constexpr (K == 2)
+        asm("v_mov_b32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_2" : "+v"(at) : "v"(w));
+    else
+        asm("v_mov_b32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3" : "+v"(at) : "v"(w));
 }
 
 __device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c)
@@ -367,32 +386,30 @@ __device__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c)
 }
 
 // lut8: the J^64 table in LDS as [256 values][16 positions] of 16-byte entries
-__device__ __forceinline__ void apply_lut8_spread(const unsigned char *__restrict__ lut8, const LaneOrder &o,
+template <int T> __device__ __forceinline__ void put_rows(LaneOrder &o, const uint32_t (&r)[4])
+{
+    if constexpr (T < 16) {
+        put_row<(T & 3)>(o.at[T], r[T >> 2]);
+        put_rows<T + 1>(o, r);
+    }
+}
+
+__device__ __forceinline__ void apply_lut8_spread(const unsigned char *__restrict__ lut8, LaneOrder &o,
                                                   uint64_t &s0, uint64_t &s1)
 {
-    uint32_t d0 = (uint32_t)s0, d1 = (uint32_t)(s0 >> 32), d2 = (uint32_t)s1, d3 = (uint32_t)(s1 >> 32);
-    // word j of the permuted state is word j ^ (l16 >> 2) of the state ...
-    uint32_t e0 = o.swap1 ? d1 : d0, e1 = o.swap1 ? d0 : d1, e2 = o.swap1 ? d3 : d2, e3 = o.swap1 ? d2 : d3;
+    const uint32_t d0 = (uint32_t)s0, d1 = (uint32_t)(s0 >> 32), d2 = (uint32_t)s1, d3 = (uint32_t)(s1 >> 32);
+    const uint32_t f0 = o.swap2 ? d2 : d0, f1 = o.swap2 ? d3 : d1, f2 = o.swap2 ? d0 : d2, f3 = o.swap2 ? d1 : d3;
     uint32_t r[4];
-    r[0] = o.swap2 ? e2 : e0;
-    r[1] = o.swap2 ? e3 : e1;
-    r[2] = o.swap2 ? e0 : e2;
-    r[3] = o.swap2 ? e1 : e3;
-    // ... with its bytes exchanged the same way
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-        r[j] = __builtin_amdgcn_perm(r[j], r[j], o.byte_select);
+    r[0] = __builtin_amdgcn_perm(f1, f0, o.select);
+    r[1] = __builtin_amdgcn_perm(f0, f1, o.select);
+    r[2] = __builtin_amdgcn_perm(f3, f2, o.select);
+    r[3] = __builtin_amdgcn_perm(f2, f3, o.select);
+    put_rows<0>(o, r);
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
     u32x4_t got[16];
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-        const uint32_t w = r[t >> 2];
-        const int k = t & 3;
-        // (byte k of w) << 8: the row of the table
-        const uint32_t row = k == 0 ? (w << 8) : k == 1 ? w : k == 2 ? (w >> 8) : (w >> 16);
-        const uint32_t at = (row & 0xFF00u) | (o.base ^ (uint32_t)(t << 4));
-        got[t] = *reinterpret_cast<const u32x4_t *>(lut8 + at);
-    }
+    for (int t = 0; t < 16; ++t)
+        got[t] = *reinterpret_cast<const u32x4_t *>(lut8 + o.at[t]);
     uint32_t acc[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -443,7 +460,7 @@ __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t 
         if ((lane >> k) & 1)
             apply_lut<4>(lut + k * 32 * 16, s0, s1);
     const unsigned char *__restrict__ step = reinterpret_cast<const unsigned char *>(lut + kLut4);  // J^64
-    const LaneOrder order = lane_order(lane);
+    LaneOrder order = lane_order(lane);
     for (int g = 0; g < kInitSteps; ++g) {
         if (first + (int64_t)g * 64 >= n)
             break;
