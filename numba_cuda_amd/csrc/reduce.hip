@@ -470,8 +470,13 @@ __global__ __launch_bounds__(kBlock) void reduce_kernel(const T *__restrict__ in
 // contiguous piece of 32 items from every "row" of S items, so a workgroup owns one of the
 // reference's warps: eight wavefronts load rows of that piece, 16 bytes per lane, two batches
 // of eight rounds in flight, and park them in LDS; 32 lanes of a ninth wavefront do nothing
-// but add down the parked rows, one chain each - 512 dependent operations per 64 KiB batch,
-// about as long as the memory takes to deliver the next one.  One launch: warp results
+// but add down the parked rows, one chain each.  That wavefront is what the kernel waits for
+// (cycle counters around its phases: busy 95 % of the time, the loading wavefronts waiting at
+// the barrier half of theirs): 32 768 rows per chain at about 1.4 instructions per row, and a
+// wavefront on its own issues an instruction every 2.5 - 3 ns on this part whatever the
+// instructions depend on (one wavefront alone in a loop of additions: 4.0 ns per dependent
+// addition, 2.9 - 3.1 ns per independent one; the same chain loop alone in a kernel: 3.9 ns
+// per row).  One launch: warp results
 // are published like the partials of reduce_kernel, the workgroup that draws the last
 // ticket does the small rest the way the reference's kernels do.
 constexpr int kOrdLoaders = 512;                 // lanes that load and park
@@ -623,10 +628,10 @@ __global__ __launch_bounds__(kOrdThreads) void reduce_ordered_kernel(const T *__
                 // way from LDS (32 dwords a set, whatever the element size)
                 constexpr int U = (32 / E) < 1 ? 1 : (32 / E);   // pairs of rows per set
                 constexpr int G = 2 * U;                          // rows per set
-                auto read = [&](Two *into, int at) {
+                auto read = [&](Two *into, int at) {     // `at` is even and not negative
 #pragma unroll
                     for (int u = 0; u < U; ++u)
-                        into[u] = pairs[at / 2 + u];
+                        into[u] = pairs[((unsigned)at >> 1) + u];
                 };
                 auto add_up = [&](const Two *from) {
 #pragma unroll
@@ -635,7 +640,62 @@ __global__ __launch_bounds__(kOrdThreads) void reduce_ordered_kernel(const T *__
                         acc = Op::apply(acc, (A)from[u].item[1]);
                     }
                 };
-                if (r + G <= count) {
+                // Four register sets take turns: the reads of a set are issued three sets (48 rows of
+                // float32) before its rows are added.  A set of reads comes back after some 70 ns, about
+                // what the sixteen dependent additions of a set take: with one set ahead the chain
+                // waits for the LDS between any two sets (196 -> 193 us for 2^28 float32; the steady
+                // loop is 77 % of the chain wavefront's time, the first and last sets of a batch the
+                // rest).  2-byte items keep two sets: their conversions need the registers.  No read
+                // in the steady loop is conditional, so every set stays in the registers it was read into.
+                if constexpr (E != 2) {
+                    if (r + 3 * G <= count) {
+                        Two s0[U], s1[U], s2[U], s3[U];
+                        const Two *__restrict__ p = pairs + ((unsigned)r >> 1);   // rows r ...: sets lie U pairs apart
+                        auto ahead = [&](Two *into, int set) {
+#pragma unroll
+                            for (int u = 0; u < U; ++u)
+                                into[u] = p[set * U + u];
+                        };
+                        ahead(s0, 0);
+                        ahead(s1, 1);
+                        ahead(s2, 2);
+                        // One step: ask for the set three ahead, wait until all reads but the twelve
+                        // youngest (three sets of four 16-byte reads) have come back - that is the set
+                        // whose turn it is - and add it up.  The explicit wait stands for the four
+                        // the compiler would place, one in front of each read's first use; the barriers
+                        // keep its scheduler from gathering the reads of several sets in one place,
+                        // which puts them right in front of their first use again.
+                        // s_waitcnt immediate: vmcnt 63 and expcnt 7 (no wait), lgkmcnt 12
+#define NBH_CHAIN_STEP(NEXT, SET, CUR)                \
+    ahead(NEXT, SET);                                  \
+    __builtin_amdgcn_sched_barrier(0);                 \
+    __builtin_amdgcn_s_waitcnt(0xCC7F);                \
+    __builtin_amdgcn_sched_barrier(0);                 \
+    add_up(CUR);                                       \
+    __builtin_amdgcn_sched_barrier(0);
+                        while (r + 7 * G <= count) {
+                            NBH_CHAIN_STEP(s3, 3, s0)
+                            NBH_CHAIN_STEP(s0, 4, s1)
+                            NBH_CHAIN_STEP(s1, 5, s2)
+                            NBH_CHAIN_STEP(s2, 6, s3)
+                            r += 4 * G;
+                            p += 4 * U;
+                        }
+#undef NBH_CHAIN_STEP
+                        const bool fourth = r + 4 * G <= count;
+                        if (fourth)
+                            ahead(s3, 3);
+                        add_up(s0);
+                        add_up(s1);
+                        add_up(s2);
+                        r += 3 * G;
+                        if (fourth) {
+                            add_up(s3);
+                            r += G;
+                        }
+                    }
+                }
+                if (r + G <= count) {                // what is left of whole sets: two sets taking turns
                     Two one[U], other[U];
                     read(one, r);
                     while (r + 3 * G <= count) {
@@ -663,54 +723,41 @@ __global__ __launch_bounds__(kOrdThreads) void reduce_ordered_kernel(const T *__
         // as soon as it has arrived (the younger one still travelling), the batch after next is
         // asked for into the registers just emptied, and the chains take the parked batch in
         // meanwhile.  One barrier per batch: whoever parks into a buffer has passed the barrier
-        // the chains reached after reading it.  The steady-state loop always asks for both
-        // batches, so that the wait before each parking is for the older eight loads only
-        // (a load that is skipped on some path would make the compiler wait for all of them);
-        // the last one to three batches are taken outside it.
+        // the chains reached after reading it.  The loading wavefronts and the chain wavefront
+        // each run a loop of their own with the same number of barriers (a wavefront is one or the
+        // other as a whole): the registers that hold batches on their way and the ones the chains
+        // read ahead into are then never live together, which one common loop would make them.
         const int64_t nb = (nrows + kBatch - 1) / kBatch;
         if (loader) {
             fetch(held[0], 0);
             fetch(held[1], kBatch);                 // rows behind the last repeat the last: harmless
-        }
-        int64_t b = 0;
-        for (; b + 3 < nb; b += 2) {
-            if (loader)
+            int64_t b = 0;
+            for (; b + 1 < nb; b += 2) {
                 park(held[0], 0);
-            __syncthreads();
-            if (loader)
-                fetch(held[0], (b + 2) * kBatch);
-            else
-                chains(0, b * kBatch);
-            if (loader)
+                __syncthreads();
+                if (b + 2 < nb)
+                    fetch(held[0], (b + 2) * kBatch);
                 park(held[1], 1);
-            __syncthreads();
-            if (loader)
-                fetch(held[1], (b + 3) * kBatch);
-            else
-                chains(1, (b + 1) * kBatch);
-        }
-        if (loader)
-            park(held[0], 0);
-        __syncthreads();
-        if (loader) {
-            if (b + 2 < nb)
-                fetch(held[0], (b + 2) * kBatch);
+                __syncthreads();
+                if (b + 3 < nb)
+                    fetch(held[1], (b + 3) * kBatch);
+            }
+            if (b < nb) {
+                park(held[0], 0);
+                __syncthreads();
+            }
         } else {
-            chains(0, b * kBatch);
-        }
-        if (b + 1 < nb) {
-            if (loader)
-                park(held[1], 1);
-            __syncthreads();
-            if (!loader)
+            int64_t b = 0;
+            for (; b + 1 < nb; b += 2) {
+                __syncthreads();
+                chains(0, b * kBatch);
+                __syncthreads();
                 chains(1, (b + 1) * kBatch);
-        }
-        if (b + 2 < nb) {
-            if (loader)
-                park(held[0], 0);
-            __syncthreads();
-            if (!loader)
-                chains(0, (b + 2) * kBatch);
+            }
+            if (b < nb) {
+                __syncthreads();
+                chains(0, b * kBatch);
+            }
         }
         if (!loader) {                              // the chain wavefront, whole: the shuffles need its lanes
 #pragma unroll
