@@ -440,11 +440,16 @@ extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce(const char *
 // One workgroup per warp of the reference: 32 chains whose items lie side by side in every
 // row of S items.  All 512 lanes load rows of 32 items into one of two LDS buffers, a batch
 // at a time, the next batch travelling while lanes 0 - 31 fold the parked one down their
-// chains.  Warp results are published like the partials above; the workgroup that draws the
+// chains.  The buffers hold the rows of a chain side by side, so that a chain reads eight of
+// its items with one or two wide LDS reads, and a batch is 512 rows of 4-byte items (2^28
+// float32 with a - b: 382 us with one 4-byte read per row and batches of 128 rows, 354 us
+// now; 8- and 16-byte items stay within 3 %); the row pitch, eight bytes more than a batch,
+// spreads the scattered stores of a wavefront over the banks.  Warp results are published like the partials above; the workgroup that draws the
 // last ticket does the small rest the way the reference's kernels do.
 constexpr int kRefWarp = 32, kRefBlock = 128, kRefMaxGrid = 64;
-constexpr int kOrdRows = (512 / (int)sizeof(T)) > 128 ? 128 : (512 / (int)sizeof(T));  // rows parked per batch
+constexpr int kOrdRows = (2048 / (int)sizeof(T)) > 512 ? 512 : (2048 / (int)sizeof(T));  // rows parked per batch
 constexpr int kOrdLoads = kOrdRows * kRefWarp / kThreads;                                // loads per lane and batch
+constexpr int kOrdPitch = kOrdRows + (sizeof(T) < 8 ? 8 / (int)sizeof(T) : 1);           // items per chain and buffer
 
 // the reference's one-block routine (:99-141) over m <= 128 values, by one thread: a full warp
 // that is not the last is a tree, the last warp a left fold, and so are the warps
@@ -478,7 +483,7 @@ extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce_ordered(cons
                                                                            nbh_u64 *__restrict__ partials,
                                                                            unsigned *__restrict__ ticket)
 {
-    __shared__ T rows[2][kOrdRows][kRefWarp];
+    __shared__ __attribute__((aligned(16))) T cols[2][kRefWarp][kOrdPitch];
     __shared__ T small[kRefBlock + 1 + kRefMaxGrid + 1];
     __shared__ bool last_block;
     const int tid = threadIdx.x;
@@ -515,7 +520,7 @@ extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce_ordered(cons
             const int buf = (int)(b & 1);
 #pragma unroll
             for (int k = 0; k < kOrdLoads; ++k)
-                rows[buf][row0 + k * kRowStep][chain] = held[k];
+                cols[buf][chain][row0 + k * kRowStep] = held[k];
             // one barrier per batch: whoever parks into a buffer next has passed the barrier
             // that the folding lanes reached after reading it
             __syncthreads();
@@ -524,22 +529,30 @@ extern "C" __global__ __launch_bounds__(512) void nbh_custom_reduce_ordered(cons
             if (tid < kRefWarp) {
                 const long long left = nrows - b * kOrdRows;
                 const int count = (int)(left < kOrdRows ? left : kOrdRows);
+                const T *__restrict__ mine = cols[buf][tid];
                 int r = 0;
-                if (b == 0) {                       // a chain starts with its first value
-                    acc = rows[buf][0][tid];
-                    r = 1;
+                if (b == 0) {                       // a chain starts with its first value ...
+                    acc = mine[0];
+                    for (r = 1; r < 8 && r < count; ++r)   // ... and goes on in steps of eight items, aligned
+                        acc = nbh_op(acc, mine[r]);
                 }
-                for (; r + 8 <= count; r += 8) {
-                    T v[8];
+                struct alignas(8) Eight { T v[8]; };         // a chain starts on an 8-byte boundary, eight items apart stay on one
+                if (r + 8 <= count) {
+                    Eight cur = *reinterpret_cast<const Eight *>(mine + r);
+                    for (; r + 16 <= count; r += 8) {
+                        const Eight next = *reinterpret_cast<const Eight *>(mine + r + 8);
+#pragma unroll
+                        for (int j = 0; j < 8; ++j)
+                            acc = nbh_op(acc, cur.v[j]);
+                        cur = next;
+                    }
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
-                        v[j] = rows[buf][r + j][tid];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-                        acc = nbh_op(acc, v[j]);
+                        acc = nbh_op(acc, cur.v[j]);
+                    r += 8;
                 }
                 for (; r < count; ++r)
-                    acc = nbh_op(acc, rows[buf][r][tid]);
+                    acc = nbh_op(acc, mine[r]);
             }
         }
         if (tid < 64) {                             // the first wavefront, whole: the shuffles need its lanes
