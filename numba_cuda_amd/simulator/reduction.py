@@ -4,7 +4,9 @@ call per element, `init` used as given (numba_cuda/numba/cuda/simulator/reductio
 from functools import reduce as _fold
 
 
-def Reduce(func):
+def Reduce(func, reference_order=None):
+    """`reference_order` (this package's own argument of the GPU mode's Reduce) is accepted and
+    has nothing to choose here: the fold has one order."""
     def reduce_wrapper(seq, res=None, init=0):
         value = _fold(func, seq, init)
         if res is None:

@@ -46,6 +46,15 @@ def test_reduce_into_a_result_array_and_other_operators():
     assert simcuda.reduce(lambda x, y: max(x, y))(simcuda.to_device(np.array([3., -1., 9., 2.])), init=-np.inf) == 9.0
 
 
+def test_reduce_takes_the_gpu_mode_constructor_arguments():
+    """Code written for the GPU mode (`Reduce(functor, reference_order=True)`) runs unchanged:
+    the left fold has one order, the argument chooses nothing."""
+    minus = lambda x, y: x - y
+    a = np.arange(10, dtype=np.float32)
+    assert simcuda.Reduce(minus, reference_order=True)(a, init=1) == sim.Reduce(minus)(a, init=1)
+    assert simcuda.Reduce(minus, reference_order=False)(a, init=1) == simcuda.reduce(minus)(a, init=1)
+
+
 # ---- arrays -------------------------------------------------------------------------------
 
 def test_to_device_owns_its_bytes_and_round_trips():
