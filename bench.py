@@ -46,7 +46,7 @@ MEASURED_TRAFFIC = {
     "reduce_f32_max": 1073819617,
     "reduce_f64_sum": 1073818517,
     "reduce_i64_sum": 2147532373,
-    "reduce_f32_sum_reference_order": 1073926486,
+    "reduce_f32_sum_reference_order": 1073951990,
     "reduce_f32_functor": 1073931926,
     "rng_uniform_f32": 4831250488,
     "rng_normal_f64": 2684020788,

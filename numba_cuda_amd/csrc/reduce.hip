@@ -643,11 +643,14 @@ __global__ __launch_bounds__(kOrdThreads) void reduce_ordered_kernel(const T *__
                 // Four register sets take turns: the reads of a set are issued three sets (48 rows of
                 // float32) before its rows are added.  A set of reads comes back after some 70 ns, about
                 // what the sixteen dependent additions of a set take: with one set ahead the chain
-                // waits for the LDS between any two sets (196 -> 193 us for 2^28 float32; the steady
+                // waits for the LDS between any two sets (196 -> 193 us for 2^28 float32, 190 us with the fixed trip count for whole batches below; the steady
                 // loop is 77 % of the chain wavefront's time, the first and last sets of a batch the
                 // rest).  2-byte items keep two sets: their conversions need the registers.  No read
                 // in the steady loop is conditional, so every set stays in the registers it was read into.
                 if constexpr (E != 2) {
+                    // a whole batch in the middle of a chain, which is what all but the first and the
+                    // last of a chain's batches are: nothing depends on `count`, the trip count is fixed
+                    const bool whole = base != 0 && count == kBatch;
                     if (r + 3 * G <= count) {
                         Two s0[U], s1[U], s2[U], s3[U];
                         const Two *__restrict__ p = pairs + ((unsigned)r >> 1);   // rows r ...: sets lie U pairs apart
@@ -673,6 +676,23 @@ __global__ __launch_bounds__(kOrdThreads) void reduce_ordered_kernel(const T *__
     __builtin_amdgcn_sched_barrier(0);                 \
     add_up(CUR);                                       \
     __builtin_amdgcn_sched_barrier(0);
+                        if (whole) {
+                            static_assert(kBatch % (4 * G) == 0 && kBatch >= 8 * G, "whole rounds of four sets");
+#pragma unroll 1
+                            for (int round = 0; round < kBatch / (4 * G) - 1; ++round) {
+                                NBH_CHAIN_STEP(s3, 3, s0)
+                                NBH_CHAIN_STEP(s0, 4, s1)
+                                NBH_CHAIN_STEP(s1, 5, s2)
+                                NBH_CHAIN_STEP(s2, 6, s3)
+                                p += 4 * U;
+                            }
+                            ahead(s3, 3);
+                            add_up(s0);
+                            add_up(s1);
+                            add_up(s2);
+                            add_up(s3);
+                            return;
+                        }
                         while (r + 7 * G <= count) {
                             NBH_CHAIN_STEP(s3, 3, s0)
                             NBH_CHAIN_STEP(s0, 4, s1)
