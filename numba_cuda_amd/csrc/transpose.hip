@@ -180,6 +180,8 @@ template <int E_, int RING_, int TC_, int PAD_, int THREADS_, int STEPS_, int SE
 // the rows above a strip, read a second time, cost less than the lost overlap did.
 // 2-byte items: 256 x 64 in two steps with 256 threads -> one step with 512
 // threads and the unguarded interior path: 8193 x 32769 214 -> 206 us, 30001 x 7001 195 -> 183.
+// 8-byte items, float64 12345 x 6789: ring 256 x 32 (half the rows read twice, half the workgroups per
+// compute unit) 234 -> 253 us, ring 128 x 64 with 512 threads 234 -> 243 us: 128 x 32 stays.
 template <int E> struct ShearOf;
 template <> struct ShearOf<2> { using type = RingCfg<2, 256, 64, 8, 512, 1>; };
 template <> struct ShearOf<4> { using type = RingCfg<4, 256, 64, 4, 512, 1>; };
