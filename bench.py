@@ -41,7 +41,7 @@ MEASURED_TRAFFIC = {
     "reduce_f32_sum": 1073804215,
     "copy_f32": 2147483648,                      # the calibration kernel itself
     "transpose_f32": 2148246600,
-    "transpose_f64": 1438988253,
+    "transpose_f64": 1349570873,
     "transpose_i16": 1073881556,
     "reduce_f32_max": 1073819617,
     "reduce_f64_sum": 1073818517,

@@ -218,15 +218,22 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
         if (logical < per * 8)
             logical = (logical % 8) * per + logical / 8;
     }
-    // kOrderPadded: the strips of a column band are counted up to a multiple of 8, so that
-    // tiles side by side (same strip, neighbouring bands) run on the same XCD, strips_pad / 8
+    // kOrderPadded: the strips of a column band are counted up to a multiple of 8, and XCD x
+    // (workgroup index mod 8) walks down the x-th run of neighbouring strips of every band.
+    // Tiles side by side (same strip, neighbouring bands) then run on the same XCD, strips_pad / 8
     // dispatches apart: the line of every input row that straddles their common edge is
-    // fetched from memory once and found in that XCD's L2 the second time, while the order
-    // in which the chip walks through the matrix stays what it was.  (float64 12345 x 6789:
-    // fetched bytes 1.62 -> 1.15 x the input; the surplus workgroups leave at once.)
+    // fetched from memory once and found in that XCD's L2 the second time.  So are the S rows
+    // above a tile, which the tile above, eight workgroups earlier on the same XCD, reads as its
+    // last ones.  The order in which the chip walks through the matrix stays what it was.
+    // (float64 12345 x 6789: fetched bytes 1.62 x the input in plain order, 1.15 x with the
+    // strips dealt to the XCDs one by one, 1.01 x with the runs - at the same 233 - 235 us, the
+    // kernel is not short of bandwidth; 8193^2 188 -> 184 us, 20001 x 5003 290 -> 288.  The surplus
+    // workgroups leave at once.)
     const int64_t strips_pad = order == kOrderPadded ? (strips_r + 7) / 8 * 8 : strips_r;
     const int64_t tile_c = logical / strips_pad;
-    const int64_t strip = logical % strips_pad;
+    int64_t strip = logical % strips_pad;
+    if (order == kOrderPadded)
+        strip = (strip % 8) * (strips_pad / 8) + strip / 8;
     if (strip >= strips_r)
         return;
     const int64_t C0 = tile_c * TC;
@@ -257,6 +264,11 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
     // float64 4099 x 20000 229 -> 243) and for 16-byte items always (8193^2 366 -> 401):
     // those keep the general path.  2-byte items gain either way (8193 x 32769 214 -> 206,
     // 10001 x 12001 88 -> 75, input rows on the grid 8193 x 32768 206 -> 205).
+    // One workgroup per tile, here for a few microseconds, is also what keeps the memory busy:
+    // the same path as a loop in as many resident workgroups as the chip holds, each asking
+    // for its next tile's loads while it reads the ring and stores, was slower on every shape
+    // (float64 12345 x 6789 234 -> 266 us, float32 16100^2 366 -> 429, int16 8193 x 32769
+    // 210 -> 279): a workgroup that ends frees its place while its stores are still on their way.
     if constexpr (Cfg::STEPS == 1 && E < 16) {
         if (lean && strip_begin >= S && strip_begin + TR < rows && C0 + TC <= cols) {
             constexpr int RPS = kThr / PPR;      // tile rows one round of the workgroup loads
