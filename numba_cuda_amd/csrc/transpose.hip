@@ -269,6 +269,11 @@ __global__ __launch_bounds__(Cfg::THREADS) void transpose_sheared(const char *__
     // for its next tile's loads while it reads the ring and stores, was slower on every shape
     // (float64 12345 x 6789 234 -> 266 us, float32 16100^2 366 -> 429, int16 8193 x 32769
     // 210 -> 279): a workgroup that ends frees its place while its stores are still on their way.
+    // Nor is it the way into LDS that costs: the tile loaded straight into LDS (eight
+    // global_load_lds_dwordx4 per lane into unpadded 256-byte rows, the packets of a row permuted by
+    // the row number so that the column reads stay free of bank conflicts; no registers held, no
+    // LDS write instructions) runs float64 12345 x 6789 in 236.6 us against 235.0, and 4099 x 20000,
+    // 8193^2, 20001 x 5003 within 0.3 % of this path.
     if constexpr (Cfg::STEPS == 1 && E < 16) {
         if (lean && strip_begin >= S && strip_begin + TR < rows && C0 + TC <= cols) {
             constexpr int RPS = kThr / PPR;      // tile rows one round of the workgroup loads
