@@ -40,9 +40,9 @@ MEASURED_TRAFFIC = {
     # fetched + written bytes per launch; each figure is derived in the profiles/ file TRAFFIC_SOURCE names
     "reduce_f32_sum": 1073804215,
     "copy_f32": 2147483648,                      # the calibration kernel itself
-    "transpose_f32": 2148246600,
+    "transpose_f32": 2147948643,
     "transpose_f64": 1349570873,
-    "transpose_i16": 1073881556,
+    "transpose_i16": 1073941648,
     "reduce_f32_max": 1073819617,
     "reduce_f64_sum": 1073818517,
     "reduce_i64_sum": 2147532373,

@@ -109,7 +109,7 @@ __device__ __forceinline__ void move_block(const char *__restrict__ in, char *__
 template <int E, bool NT, typename Shape = ShapeOf<E>>
 __global__ __launch_bounds__(64 * Shape::WR * Shape::WC) void transpose_packets(
     const char *__restrict__ in, char *__restrict__ out, int64_t rows, int64_t cols, int64_t in_s0, int64_t out_s0,
-    int64_t tiles_r)
+    int64_t tiles_r, bool diagonal)
 {
     constexpr int V = 16 / E;
     constexpr int WT = 8 * V;  // wavefront tile edge, in items
@@ -119,7 +119,20 @@ __global__ __launch_bounds__(64 * Shape::WR * Shape::WC) void transpose_packets(
     // consecutive workgroups go down the input rows = along the output rows
     int64_t tile_c = (int64_t)blockIdx.x / tiles_r;
     const int64_t tile_r = (int64_t)blockIdx.x % tiles_r;
-    if (E == 2) {
+    if (diagonal) {
+        // Output rows exactly 32 KiB apart, input rows a power of two of at most that: the
+        // workgroups that run together (consecutive ones, going down the input rows) each take
+        // the next column band as well, so that they write to different output rows.
+        // Measured, us, bands in order (two passes for 2-byte items) -> diagonal, with the two
+        // pitches in KiB: int16 16384^2 (32/32) 211 -> 190, 16384 x 8192 (16/32) 104 -> 96,
+        // 16384 x 4096 (8/32) 52.8 -> 48.1; float32 8192^2 (32/32) 97.7 -> 93.3, 8192 x 4096
+        // (16/32) 49.3 -> 47.4; float64 4096^2 (32/32) 47.1 -> 44.9.  No other pair of pitches
+        // gains on every shape tried: output rows 64 KiB apart lose 4 - 9 % with input rows
+        // as far apart (float32 16384^2 352 -> 385) and win or lose with shorter ones (float32
+        // 16384 x 8192 205 -> 191, int16 32768 x 16384 370 -> 402); pitches that are no
+        // powers of two lose (float32 16000^2 353 -> 423, 12000 x 8192 141 -> 151).
+        tile_c = (tile_c + tile_r) % ((int64_t)gridDim.x / tiles_r);
+    } else if (E == 2) {
         // 2-byte items: the column bands are walked in two passes, even bands first, then odd
         // ones, so that bands side by side are not in flight together.  Measured, bands in
         // order -> two passes, us: 8192 x 32768 191.3 -> 188.1, 32768 x 8192 216.8 -> 209.9,
@@ -538,12 +551,15 @@ int launch_packets(const void *in, void *out, int64_t rows, int64_t cols, int64_
     const double moved = 2.0 * (double)rows * (double)cols * E;
     const double threshold = E == 4 ? 0.75 * (1u << 30) : 1.5 * (1u << 30);
     const unsigned throttle = ((E == 2 || E == 4 || E == 8) && moved >= threshold) ? 54000u : 0u;
+    // the order in which the workgroups take the tiles, by the two pitches (measurements at the kernel)
+    const bool diagonal = (E == 2 || E == 4 || E == 8) && out_s0 == 32768 && in_s0 > 0 && in_s0 <= 32768 &&
+                          (in_s0 & (in_s0 - 1)) == 0;
     if (mix % 128 == 0)
         hipLaunchKernelGGL((transpose_packets<E, true, Shape>), grid, block, throttle, stream, (const char *)in,
-                           (char *)out, rows, cols, in_s0, out_s0, tiles_r);
+                           (char *)out, rows, cols, in_s0, out_s0, tiles_r, diagonal);
     else
         hipLaunchKernelGGL((transpose_packets<E, false, Shape>), grid, block, throttle, stream, (const char *)in,
-                           (char *)out, rows, cols, in_s0, out_s0, tiles_r);
+                           (char *)out, rows, cols, in_s0, out_s0, tiles_r, diagonal);
     return nbh_launch_status();
 }
 

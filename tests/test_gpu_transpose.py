@@ -182,6 +182,21 @@ def test_random_shapes_pitches_and_offsets(seed):
         assert _same_bytes(dst_full.copy_to_host(), want), (dtype, rows, cols, pad_in, off_in, pad_out, off_out)
 
 
+@pytest.mark.parametrize("dtype,rows,cols", [(np.int16, 16384, 256), (np.int16, 16384, 1100), (np.uint16, 16384, 4096),
+                                             (np.float32, 8192, 128), (np.float32, 8192, 2048), (np.uint32, 8192, 8192),
+                                             (np.float64, 4096, 64), (np.float64, 4096, 1000), (np.int64, 4096, 4096)])
+def test_output_rows_32_kib_apart(dtype, rows, cols):
+    """Output rows exactly 32 KiB apart: with input rows a power of two of at most that the
+    workgroups take the tiles in diagonal order (several column bands, one band, bands whose
+    number does not divide the rows' tiles), otherwise in the plain one."""
+    dtype = np.dtype(dtype)
+    _say("transpose 32 KiB output pitch", dtype, rows, cols)
+    rng = np.random.default_rng(rows + cols)
+    a = rng.integers(0, 256, (rows, cols * dtype.itemsize), dtype=np.uint8).view(dtype)
+    got = transpose(cuda.to_device(a)).copy_to_host()
+    assert _same_bytes(got, a.T)
+
+
 # ---- full-size matrices, seed 2 --------- ------------------------------------------------
 
 def test_fullsize_float32_16384_square():
