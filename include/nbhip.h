@@ -54,6 +54,10 @@ enum nbh_op { NBH_ADD = 0, NBH_MUL = 1, NBH_MAX = 2, NBH_MIN = 3, NBH_AND = 4, N
 /* ---- library / device ---------------------------------------------------- */
 
 int nbh_version(void);
+/* cudadrv/driver.py:410-418 Driver.get_version, cudadrv/runtime.py:15-24 Runtime.get_version:
+ * the versions of the HIP driver and runtime as HIP encodes them, major * 10 000 000 +
+ * minor * 100 000 + patch.  Needs no device. */
+int nbh_hip_versions(int *driver_version, int *runtime_version);
 
 /* cudadrv/driver.py:245-419 Driver (error checking): name / text of an error code */
 const char *nbh_error_name(int code);

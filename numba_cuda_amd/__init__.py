@@ -39,6 +39,7 @@ else:
                                                ManagedMemory, MemoryPointer, MappedMemory,
                                                PinnedMemory, MemoryInfo, set_memory_manager)
     from numba_cuda_amd.cudadrv.devicearray import DeviceNDArray, DeviceRecord  # noqa: F401
+    from numba_cuda_amd.cudadrv.runtime import runtime  # noqa: F401
     from numba_cuda_amd.api import *  # noqa: F401,F403
     from numba_cuda_amd.api import (_auto_device, _contiguous_strides_like_array, _order_like_array,  # noqa: F401
                                     current_context, gpus, require_context)

@@ -23,6 +23,7 @@ P = ctypes.POINTER
 # name -> (restype, argtypes); must list every symbol include/nbhip.h declares
 SIGNATURES = {
     "nbh_version": (c_int, []),
+    "nbh_hip_versions": (c_int, [P(c_int), P(c_int)]),
     "nbh_error_name": (c_char_p, [c_int]),
     "nbh_error_string": (c_char_p, [c_int]),
     "nbh_device_count": (c_int, [P(c_int)]),

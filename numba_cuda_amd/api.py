@@ -313,6 +313,13 @@ def cuda_error():
     return driver.driver.initialization_error
 
 
+def is_supported_version():
+    """True if the HIP runtime is a version this package is tested with (reference:
+    device_init.py:128-143; other versions may still work)."""
+    from numba_cuda_amd.cudadrv.runtime import runtime
+    return runtime.is_supported_version()
+
+
 def is_float16_supported():
     return True
 

@@ -11,6 +11,16 @@ extern "C" {
 
 int nbh_version(void) { return NBH_VERSION; }
 
+int nbh_hip_versions(int *driver_version, int *runtime_version)
+{
+    if (!driver_version || !runtime_version)
+        return (int)hipErrorInvalidValue;
+    hipError_t e = hipDriverGetVersion(driver_version);
+    if (e == hipSuccess)
+        e = hipRuntimeGetVersion(runtime_version);
+    return (int)e;
+}
+
 const char *nbh_error_name(int code) { return hipGetErrorName((hipError_t)code); }
 const char *nbh_error_string(int code) { return hipGetErrorString((hipError_t)code); }
 

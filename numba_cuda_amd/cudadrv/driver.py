@@ -188,7 +188,14 @@ class Driver:
         return [self.get_device(i) for i in range(self.get_device_count())]
 
     def get_version(self):
-        return (self.lib.nbh_version(), 0)
+        """The HIP driver's version as (major, minor); reference :410-418."""
+        return self.hip_versions()[0]
+
+    def hip_versions(self):
+        """((major, minor) of the HIP driver, (major, minor) of the HIP runtime)."""
+        drv, rt = c_int(0), c_int(0)
+        self.nbh_hip_versions(byref(drv), byref(rt))
+        return tuple((v // 10000000, v // 100000 % 100) for v in (drv.value, rt.value))
 
     # --- the calling thread's active context (reference :387-407; HIP has one implicit
     # context per device, so "pushed" contexts are a per-thread list kept here)

@@ -114,5 +114,14 @@ def auto_device_helper(cuda):
     assert again is dev and not fresh
 
 
+def driver_and_runtime_versions(cuda):
+    # cudadrv/driver.py:410-418, 2732-2736; cudadrv/runtime.py:15-33; device_init.py:128-143
+    from numba_cuda_amd.cudadrv import runtime
+    major, minor = driver.get_version()
+    assert major >= 6 and 0 <= minor < 100
+    assert runtime.get_version() == cuda.runtime.get_version() and runtime.get_version()[0] >= 6
+    assert cuda.is_supported_version() is True
+
+
 ALL = [select_device_in_fresh_threads, select_and_close_repeatedly, gpus_list_and_memory_info,
-       active_context_and_push_pop, auto_device_helper]
+       active_context_and_push_pop, auto_device_helper, driver_and_runtime_versions]

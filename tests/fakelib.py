@@ -45,6 +45,11 @@ class FakeLib:
     def nbh_version(self):
         return 1
 
+    def nbh_hip_versions(self, driver_version, runtime_version):
+        self._out(driver_version, 70226015)      # 7.2.26015
+        self._out(runtime_version, 70226015)
+        return 0
+
     def nbh_error_name(self, code):
         return {2: b"hipErrorOutOfMemory", 1: b"hipErrorInvalidValue", 600: b"hipErrorNotReady"}.get(
             code, b"hipErrorUnknown")

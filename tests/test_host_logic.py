@@ -52,6 +52,20 @@ def test_library_loads_without_a_gpu_and_reports_errors_by_name():
     assert lib.nbh_transpose(None, None, 0, 5, 4, 4, 4, 4, 4, None) == 0      # empty: nothing to do
 
 
+def test_versions_of_driver_and_runtime(fake_gpu):
+    """Driver.get_version / runtime.get_version / is_supported_version (reference
+    cudadrv/driver.py:410-418, cudadrv/runtime.py:15-33, device_init.py:128-143)."""
+    import numba_cuda_amd as cuda
+    from numba_cuda_amd.cudadrv import driver, runtime
+    assert driver.get_version() == (7, 2)
+    assert runtime.get_version() == (7, 2) == cuda.runtime.get_version()
+    assert cuda.is_supported_version() is True
+    fake_gpu.nbh_hip_versions = lambda d, r: (fake_gpu._out(d, 50700000), fake_gpu._out(r, 50700000), 0)[2]
+    driver.driver.__dict__.pop("nbh_hip_versions", None)      # the cached wrapper of the entry point
+    assert runtime.get_version() == (5, 7)
+    assert cuda.is_supported_version() is False
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libnbhip.so"))
