@@ -128,11 +128,10 @@ template <typename Tab> BM_FN double log_positive_f32(float u, Tab tab)
     p = fma_const(r, p, -1.0 / 4.0);
     p = fma_const(r, p, 1.0 / 3.0);
     p = __builtin_fma(r, p, -0.5);
-    p = (r * r) * p;
     const double ln2_hi = 0x1.62e42feep-1;             // 32 bits of ln 2
     const double ln2_lo = 0x1.a39ef35793c76p-33;       // ln 2 - ln2_hi
     const double hi = __builtin_fma(fe, ln2_hi, tab->t_hi[j]);  // exact
-    const double lo = __builtin_fma(fe, ln2_lo, tab->t_lo[j]) + p;
+    const double lo = __builtin_fma(r * r, p, __builtin_fma(fe, ln2_lo, tab->t_lo[j]));
     return hi + (r + lo);                              // the small terms first
 }
 
@@ -142,10 +141,22 @@ template <typename Tab> BM_FN double bm_log_f32(float u, Tab tab)
     return (u == 0.0f) ? -HUGE_VAL : v;
 }
 
+// What the generators use: the logarithm rounded to float32.  The case u == 0 is sorted out
+// after the rounding, on one 32-bit word instead of two.
+template <typename Tab> BM_FN float bm_log_f32_rounded(float u, Tab tab)
+{
+    const float v = (float)log_positive_f32(u, tab);
+    return (u == 0.0f) ? -HUGE_VALF : v;
+}
+
 // ---- cosine ------------------------------------------------------------------------
 // x = n * pi/2 + (y0 + y1), n = 0..4, |y0| <= pi/4 (+ a rounding's worth), with pi/2
 // carried to 119 bits in three pieces so that y0 + y1 is good to 2^-65 relative even
-// for x = RN(pi/2), where everything but 6e-17 cancels.  On [-pi/4, pi/4], with
+// for x = RN(pi/2), where everything but 6e-17 cancels.  y0 is the difference rounded once and y1
+// what it lacks: below 2^-53 of y0 except where the difference cancels, and small against y0 there
+// too, which is all the two formulas below ask of the pair (a y0 that also absorbs the third piece,
+// as a general-purpose reduction makes it, costs four more operations and changes nothing the
+// sweeps see).  On [-pi/4, pi/4], with
 // z = y0^2 (coefficients S1..S6, C1..C6: the minimax sets of fdlibm's __kernel_sin /
 // __kernel_cos),
 //     sin(y0 + y1) = y0 + [ y0 z  (S1 + z (S2 + ... z S6)) + y1 (1 - z/2) ]
@@ -163,11 +174,9 @@ template <typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
     const double fn = __builtin_rint(x * inv_pio2);
     const int n = (int)fn;
     const double t = __builtin_fma(-fn, pio2_1, x);    // exact: fn * pio2_1 has 36 bits
-    const double w = fn * pio2_2;                      // exact
-    const double r = t - w;
-    const double w2 = __builtin_fma(fn, pio2_2t, -((t - r) - w));
-    const double y0 = r - w2;
-    const double y1 = (r - y0) - w2;
+    const double y0 = __builtin_fma(-fn, pio2_2, t);   // fn * pio2_2 is exact too: one rounding, of t - fn * pio2_2
+    // what that rounding lost (t - y0 is exact and so is the fused operation), less the third piece
+    const double y1 = __builtin_fma(-fn, pio2_2t, __builtin_fma(-fn, pio2_2, t - y0));
 
     const bool odd = (n & 1) != 0;                     // odd quadrant: -+sin, even: +-cos
     auto k = &tab->trig[n & 1][0];                     // S6..S1 : C6..C1
@@ -177,8 +186,7 @@ template <typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
     asm("" : "+v"(k));
 #endif
     const double z = y0 * y0;
-    const double hz = 0.5 * z;
-    const double wc = 1.0 - hz;
+    const double wc = __builtin_fma(-0.5, z, 1.0);     // 1 - z/2, one rounding (z/2 is exact)
     double q = __builtin_fma(z, k[0], k[1]);
     q = __builtin_fma(z, q, k[2]);
     q = __builtin_fma(z, q, k[3]);
@@ -186,7 +194,8 @@ template <typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
     q = __builtin_fma(z, q, k[5]);
     const double factor = z * (odd ? y0 : z);
     const double tail_sin = y1 * wc;
-    const double tail_cos = __builtin_fma(-y0, y1, (1.0 - wc) - hz);
+    // (1 - wc) - z/2: what the rounding of wc lost; 1 - wc is exact, so this is too
+    const double tail_cos = __builtin_fma(-y0, y1, __builtin_fma(-0.5, z, 1.0 - wc));
     const double tail = odd ? tail_sin : tail_cos;
     const double base = odd ? y0 : wc;
     const double pick = base + __builtin_fma(factor, q, tail);
@@ -209,7 +218,10 @@ template <typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
 // estimate is good to 2^-26 or so, the coupled step squares that, and the correction -
 // the residual a - g^2 is exact in the fused operation - leaves an error near 2^-100 before
 // the one rounding.  (A second correction, as the general routine has it, changes none of
-// the float64 normals over all 260 million values the first uniform can take.)
+// the float64 normals over all 260 million values the first uniform can take.  Leaving h
+// as the estimate gave it would save an operation and leave an error near 2^-77: enough to
+// move the last bit of some thirty of those values.)
+// Zero and +infinity, where the estimate is infinite or zero, are told by one class test.
 BM_FN double bm_sqrt_pos(double a)
 {
 #ifdef __HIP_DEVICE_COMPILE__
@@ -221,7 +233,8 @@ BM_FN double bm_sqrt_pos(double a)
     h = __builtin_fma(h, r, h);
     const double d = __builtin_fma(-g, g, a);
     g = __builtin_fma(d, h, g);
-    return (a == 0.0 || a == HUGE_VAL) ? a : g;
+    constexpr int kZeroOrPlusInfinity = 0x020 | 0x040 | 0x200;  // -0, +0, +infinity
+    return __builtin_amdgcn_class(a, kZeroOrPlusInfinity) ? a : g;
 #else
     return std::sqrt(a);
 #endif

@@ -523,7 +523,7 @@ struct NormalF32 {
         const float u1 = UniformF32::draw(s0, s1);
         const float u2 = UniformF32::draw(s0, s1);
         const float two_pi = 6.283185307179586f;
-        const float lg = (float)bm::bm_log_f32(u1, tab);
+        const float lg = bm::bm_log_f32_rounded(u1, tab);
         const float r = sqrtf(-2.0f * lg);
         const float c = (float)bm::bm_cos_2pi((double)(two_pi * u2), tab);
         return r * c;
@@ -539,7 +539,7 @@ struct NormalF64 {
         const float u1 = UniformF32::draw(s0, s1);
         const float u2 = UniformF32::draw(s0, s1);
         const double two_pi = 6.283185307179586;
-        const float lg = (float)bm::bm_log_f32(u1, tab);
+        const float lg = bm::bm_log_f32_rounded(u1, tab);
         const double r = bm::bm_sqrt_pos(-2.0 * (double)lg);
         const double c = bm::bm_cos_2pi(two_pi * (double)u2, tab);
         return r * c;
