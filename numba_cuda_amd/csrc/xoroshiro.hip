@@ -10,10 +10,11 @@
 //   * J^first (bits >= 12 of the index, the same vector in every lane): the 64
 //     lanes split the 128 columns between them and XOR-reduce across the
 //     wavefront - about 40 instructions per product instead of 1150;
-//   * J^l, l < 64 (a different matrix subset per lane) and the J^64 step (a
-//     different vector per lane): lookup tables in LDS, 4 bits of the vector per
-//     lookup for J^1..J^32 and 8 bits per lookup for J^64 (112 KiB per workgroup,
-//     one 1024-thread workgroup per compute unit);
+//   * J^l, l < 64 (the same vector in every lane, a different matrix per lane): byte
+//     tables of all 64 matrices in global memory, laid out [position][byte][lane], so that
+//     each of the sixteen look-ups of a wavefront is one 1 KiB run (4 MiB per device);
+//   * the J^64 step (a different vector per lane): byte tables in LDS, sixteen look-ups
+//     of 16 bytes per step (64 KiB per 1024-thread workgroup);
 //   * small arrays skip the tables and use masked XORs over all 128 columns.
 //
 // Draws.  Each lane owns one generator whose 128-bit state stays in registers.
@@ -64,15 +65,16 @@ inline U128 jump_h(U128 s)
 constexpr int kPowers = 64;
 // table[k][c] = column c of J^(2^k): the image of the state with only bit c set
 // (bits 0..63 live in s0, bits 64..127 in s1).
-constexpr int kLaneTables = 6;  // J^1 .. J^32, indexed by 4 bits of the vector
 struct JumpTable {
     U128 col[kPowers][128];
-    // lut4[k][p][v]: XOR of columns 4p+b of J^(2^k) over the set bits b of v
-    U128 lut4[kLaneTables][32][16];
     // lut8[p][v]: XOR of columns 8p+b of J^64 over the set bits b of v
     U128 lut8[16][256];
+    // lane8[p][v][l]: XOR of columns 8p+b of J^l over the set bits b of v, l = 0 .. 63 (4 MiB):
+    // J^l applied to a vector is the XOR of sixteen entries, and when the 64 lanes of a wavefront
+    // hold the SAME vector, lane l wanting J^l of it, entry (p, v) of all lanes is one 1 KiB run
+    U128 lane8[16][256][64];
 };
-constexpr int kLutEntries = kLaneTables * 32 * 16 + 16 * 256;  // lut4 and lut8 are contiguous
+constexpr int kLutEntries = 16 * 256;
 
 inline U128 apply_h(const U128 *m, U128 v)
 {
@@ -103,17 +105,23 @@ const JumpTable &jump_table()
         for (int k = 1; k < kPowers; ++k)  // square: column c of M*M is M applied to column c of M
             for (int c = 0; c < 128; ++c)
                 t->col[k][c] = apply_h(t->col[k - 1], t->col[k - 1][c]);
-        for (int k = 0; k < kLaneTables; ++k)
-            for (int p = 0; p < 32; ++p)
-                for (int v = 0; v < 16; ++v) {
-                    U128 x = {0, 0};
-                    for (int b = 0; b < 4; ++b)
-                        if ((v >> b) & 1) {
-                            x.s0 ^= t->col[k][4 * p + b].s0;
-                            x.s1 ^= t->col[k][4 * p + b].s1;
-                        }
-                    t->lut4[k][p][v] = x;
+        // the columns of J^l, l = 0 .. 63, one power after the other, and their byte tables
+        {
+            U128 power[128];
+            for (int c = 0; c < 128; ++c)
+                power[c] = U128{c < 64 ? (1ull << c) : 0, c < 64 ? 0 : (1ull << (c - 64))};
+            for (int l = 0; l < 64; ++l) {
+                for (int p = 0; p < 16; ++p) {
+                    t->lane8[p][0][l] = U128{0, 0};
+                    for (int v = 1; v < 256; ++v) {
+                        const U128 rest = t->lane8[p][v & (v - 1)][l], col = power[8 * p + __builtin_ctz(v)];
+                        t->lane8[p][v][l] = U128{rest.s0 ^ col.s0, rest.s1 ^ col.s1};
+                    }
                 }
+                for (int c = 0; c < 128; ++c)
+                    power[c] = apply_h(t->col[0], power[c]);
+            }
+        }
         for (int p = 0; p < 16; ++p)
             for (int v = 0; v < 256; ++v) {
                 U128 x = {0, 0};
@@ -130,7 +138,7 @@ const JumpTable &jump_table()
 }
 
 // Device copy of the table, one per device, made on first use and kept for the
-// life of the process (240 KiB: matrix columns and lookup tables).
+// life of the process (4.2 MiB: matrix columns and lookup tables).
 int device_table(const U128 **out)
 {
     constexpr int kMaxDev = 64;
@@ -314,22 +322,6 @@ __device__ __forceinline__ void apply_shared(const U128 *__restrict__ m, int lan
 
 typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
 
-// r = M * (s0, s1) from a table indexed by BITS bits of the vector at a time.
-template <int BITS>
-__device__ __forceinline__ void apply_lut(const u64x2_t *__restrict__ lut, uint64_t &s0, uint64_t &s1)
-{
-    constexpr int N = 1 << BITS;       // entries per position
-    constexpr int HALF = 64 / BITS;    // positions per 64-bit word
-    u64x2_t r = {0, 0};
-#pragma unroll
-    for (int p = 0; p < HALF; ++p) {
-        r ^= lut[p * N + (int)((s0 >> (p * BITS)) & (N - 1))];
-        r ^= lut[(HALF + p) * N + (int)((s1 >> (p * BITS)) & (N - 1))];
-    }
-    s0 = r.x;
-    s1 = r.y;
-}
-
 constexpr int kTabBlock = 1024;
 constexpr int64_t kTablesFrom = 1 << 18;  // below this the table load outweighs its benefit
 
@@ -429,38 +421,71 @@ __device__ __forceinline__ void apply_lut8_spread(const unsigned char *__restric
 __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t *__restrict__ states, int64_t n,
                                                                        uint64_t b0, uint64_t b1,
                                                                        const U128 *__restrict__ table,
-                                                                       const u64x2_t *__restrict__ lut_global)
+                                                                       const u64x2_t *__restrict__ lut_global,
+                                                                       const u64x2_t *__restrict__ lane_global)
 {
-    // 112 KiB: lut4[6][32][16] as it comes, then lut8 transposed to [256 values][16 positions]
+    // 64 KiB: the byte tables of J^64, transposed to [256 values][16 positions]
     __shared__ u64x2_t lut[kLutEntries];
-    constexpr int kLut4 = kLaneTables * 32 * 16;
-    for (int i = threadIdx.x; i < kLutEntries; i += kTabBlock) {
-        const u64x2_t v = lut_global[i];
-        if (i < kLut4) {
-            lut[i] = v;
-        } else {
-            const int j = i - kLut4;  // lut8[p][value] in global memory
-            lut[kLut4 + (j & 255) * 16 + (j >> 8)] = v;
-        }
-    }
-    __syncthreads();
+    for (int i = threadIdx.x; i < kLutEntries; i += kTabBlock)
+        lut[(i & 255) * 16 + (i >> 8)] = lut_global[i];  // lut8[p][value] in global memory
 
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * (kTabBlock / 64) + (threadIdx.x >> 6);
     const int64_t first = wave * (64 * kInitSteps);
+    uint64_t s0 = b0, s1 = b1;
+    if (first < n) {
+        const uint64_t hi = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 6)) |
+                            ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 38)) << 32);
+        for (int k = 6; k < kPowers; ++k)
+            if ((hi >> (k - 6)) & 1)
+                apply_shared(table + (size_t)k * 128, lane, s0, s1);
+        // J^lane: every lane still holds the same vector, so byte p of it picks, for all lanes
+        // at once, one 1 KiB run of the table [position][byte][lane]: sixteen coalesced loads
+        // and their XOR, where six conditional 128 x 128 products through 4-bit tables in LDS
+        // cost 1200 vector instructions and 48 KiB of LDS (2^24 states: 77.4 -> 71.8 us per launch)
+        const uint64_t u0 = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)s0) |
+                            ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(s0 >> 32)) << 32);
+        const uint64_t u1 = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)s1) |
+                            ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(s1 >> 32)) << 32);
+        typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+        u32x4_t part[16];
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+            const int byte = (int)(((p < 8 ? u0 : u1) >> (8 * (p & 7))) & 255);
+            part[p] = *reinterpret_cast<const u32x4_t *>(lane_global + ((size_t)(p * 256 + byte) * 64 + lane));
+        }
+        uint32_t acc[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint32_t a = xor3(part[0][c], part[1][c], part[2][c]);
+            a = xor3(a, part[3][c], part[4][c]);
+            a = xor3(a, part[5][c], part[6][c]);
+            a = xor3(a, part[7][c], part[8][c]);
+            a = xor3(a, part[9][c], part[10][c]);
+            a = xor3(a, part[11][c], part[12][c]);
+            a = xor3(a, part[13][c], part[14][c]);
+            acc[c] = a ^ part[15][c];
+        }
+        s0 = ((uint64_t)acc[1] << 32) | acc[0];
+        s1 = ((uint64_t)acc[3] << 32) | acc[2];
+    }
+    __syncthreads();
     if (first >= n)
         return;
-    uint64_t s0 = b0, s1 = b1;
-    const uint64_t hi = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 6)) |
-                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 38)) << 32);
-    for (int k = 6; k < kPowers; ++k)
-        if ((hi >> (k - 6)) & 1)
-            apply_shared(table + (size_t)k * 128, lane, s0, s1);
-    for (int k = 0; k < kLaneTables; ++k)
-        if ((lane >> k) & 1)
-            apply_lut<4>(lut + k * 32 * 16, s0, s1);
-    const unsigned char *__restrict__ step = reinterpret_cast<const unsigned char *>(lut + kLut4);  // J^64
+    const unsigned char *__restrict__ step = reinterpret_cast<const unsigned char *>(lut);  // J^64
     LaneOrder order = lane_order(lane);
+    if (first + 64 * kInitSteps <= n) {  // a whole run: nothing to test on the way
+        u64x2_t *dst = reinterpret_cast<u64x2_t *>(states + 2 * (first + lane));
+#pragma unroll 1
+        for (int g = 0; g < kInitSteps - 1; ++g) {
+            const u64x2_t v = {s0, s1};
+            dst[(int64_t)g * 64] = v;
+            apply_lut8_spread(step, order, s0, s1);
+        }
+        const u64x2_t v = {s0, s1};
+        dst[(int64_t)(kInitSteps - 1) * 64] = v;
+        return;
+    }
     for (int g = 0; g < kInitSteps; ++g) {
         if (first + (int64_t)g * 64 >= n)
             break;
@@ -1169,8 +1194,9 @@ int nbh_xoro_init_states(void *states, int64_t n, uint64_t seed, uint64_t subseq
         if (grid > 0x7fffffffLL)
             return (int)hipErrorInvalidValue;
         const u64x2_t *lut = reinterpret_cast<const u64x2_t *>(dtable + (size_t)kPowers * 128);
+        const u64x2_t *lanes = lut + kLutEntries;
         hipLaunchKernelGGL(init_states_tables_kernel, dim3((unsigned)grid), dim3(kTabBlock), 0, hs,
-                           (uint64_t *)states, n, base.s0, base.s1, dtable, lut);
+                           (uint64_t *)states, n, base.s0, base.s1, dtable, lut, lanes);
         return nbh_launch_status();
     }
     const int64_t per_block = (int64_t)(kInitBlock / 64) * 64 * kInitSteps;
