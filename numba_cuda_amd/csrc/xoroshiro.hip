@@ -15,7 +15,8 @@
 //     each of the sixteen look-ups of a wavefront is one 1 KiB run (4 MiB per device);
 //   * the J^64 step (a different vector per lane): byte tables in LDS, sixteen look-ups
 //     of 16 bytes per step (64 KiB per 1024-thread workgroup);
-//   * small arrays skip the tables and use masked XORs over all 128 columns.
+// The number of steps a wavefront makes is chosen at launch: small arrays are spread over
+// many wavefronts of few steps (a single step needs no table in LDS at all).
 //
 // Draws.  Each lane owns one generator whose 128-bit state stays in registers.
 // The reference's layout out[t*count + i] gives every lane its own run of `count`
@@ -239,59 +240,7 @@ __device__ __forceinline__ uint64_t next_d(uint64_t &s0, uint64_t &s1)
     return r;
 }
 
-// r = M * (s0, s1) over GF(2); m is wavefront-uniform, so its columns come in
-// through scalar loads.
-__device__ __forceinline__ void apply_d(const U128 *__restrict__ m, uint64_t &s0, uint64_t &s1)
-{
-    uint64_t r0 = 0, r1 = 0;
-#pragma unroll 8
-    for (int b = 0; b < 64; ++b) {
-        const uint64_t m0 = 0 - ((s0 >> b) & 1);
-        const uint64_t m1 = 0 - ((s1 >> b) & 1);
-        r0 ^= (m[b].s0 & m0) ^ (m[64 + b].s0 & m1);
-        r1 ^= (m[b].s1 & m0) ^ (m[64 + b].s1 & m1);
-    }
-    s0 = r0;
-    s1 = r1;
-}
-
-constexpr int kInitBlock = 256;
-constexpr int kInitSteps = 64;  // consecutive 64-state groups produced by one wavefront
-
-__global__ __launch_bounds__(kInitBlock) void init_states_kernel(uint64_t *__restrict__ states, int64_t n,
-                                                                 uint64_t b0, uint64_t b1,
-                                                                 const U128 *__restrict__ table)
-{
-    const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * (kInitBlock / 64) + (threadIdx.x >> 6);
-    const int64_t first = wave * (64 * kInitSteps);  // first state index of this wavefront
-    if (first >= n)
-        return;
-    uint64_t s0 = b0, s1 = b1;
-    // J^first: every bit of `first` below 6 is zero; the rest is uniform
-    const uint64_t hi = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 6)) |
-                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 38)) << 32);
-    for (int k = 6; k < kPowers; ++k)
-        if ((hi >> (k - 6)) & 1)
-            apply_d(table + (size_t)k * 128, s0, s1);
-    // J^lane
-    for (int k = 0; k < 6; ++k)
-        if ((lane >> k) & 1)
-            apply_d(table + (size_t)k * 128, s0, s1);
-    const U128 *__restrict__ step = table + (size_t)6 * 128;  // J^64
-    for (int g = 0; g < kInitSteps; ++g) {
-        const int64_t idx = first + (int64_t)g * 64 + lane;
-        if (first + (int64_t)g * 64 >= n)
-            break;
-        if (idx < n) {
-            typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
-            u64x2 v = {s0, s1};
-            *reinterpret_cast<u64x2 *>(states + 2 * idx) = v;
-        }
-        if (g + 1 < kInitSteps)
-            apply_d(step, s0, s1);
-    }
-}
+constexpr int kInitSteps = 64;  // consecutive 64-state groups produced by one wavefront, at most
 
 // XOR of a value over the 64 lanes, returned in every lane.
 __device__ __forceinline__ uint32_t wave_xor32(uint32_t v)
@@ -323,7 +272,6 @@ __device__ __forceinline__ void apply_shared(const U128 *__restrict__ m, int lan
 typedef uint64_t u64x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kTabBlock = 1024;
-constexpr int64_t kTablesFrom = 1 << 18;  // below this the table load outweighs its benefit
 
 // One application of J^64 to every lane's own state, 16 look-ups of 8 bits each, WITHOUT bank
 // conflicts.  A wavefront's lanes hold unrelated states, so look-ups into one table hit random
@@ -422,16 +370,20 @@ __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t 
                                                                        uint64_t b0, uint64_t b1,
                                                                        const U128 *__restrict__ table,
                                                                        const u64x2_t *__restrict__ lut_global,
-                                                                       const u64x2_t *__restrict__ lane_global)
+                                                                       const u64x2_t *__restrict__ lane_global,
+                                                                       int steps)
 {
-    // 64 KiB: the byte tables of J^64, transposed to [256 values][16 positions]
+    // `steps` groups of 64 consecutive states per wavefront (1 .. kInitSteps, the host's choice:
+    // small arrays are spread over many wavefronts of few steps).  64 KiB: the byte tables of
+    // J^64, transposed to [256 values][16 positions]; not needed for a single step.
     __shared__ u64x2_t lut[kLutEntries];
-    for (int i = threadIdx.x; i < kLutEntries; i += kTabBlock)
-        lut[(i & 255) * 16 + (i >> 8)] = lut_global[i];  // lut8[p][value] in global memory
+    if (steps > 1)
+        for (int i = threadIdx.x; i < kLutEntries; i += kTabBlock)
+            lut[(i & 255) * 16 + (i >> 8)] = lut_global[i];  // lut8[p][value] in global memory
 
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * (kTabBlock / 64) + (threadIdx.x >> 6);
-    const int64_t first = wave * (64 * kInitSteps);
+    const int64_t first = wave * (64 * (int64_t)steps);
     uint64_t s0 = b0, s1 = b1;
     if (first < n) {
         const uint64_t hi = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(first >> 6)) |
@@ -474,19 +426,19 @@ __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t 
         return;
     const unsigned char *__restrict__ step = reinterpret_cast<const unsigned char *>(lut);  // J^64
     LaneOrder order = lane_order(lane);
-    if (first + 64 * kInitSteps <= n) {  // a whole run: nothing to test on the way
+    if (first + 64 * (int64_t)steps <= n) {  // a whole run: nothing to test on the way
         u64x2_t *dst = reinterpret_cast<u64x2_t *>(states + 2 * (first + lane));
 #pragma unroll 1
-        for (int g = 0; g < kInitSteps - 1; ++g) {
+        for (int g = 0; g < steps - 1; ++g) {
             const u64x2_t v = {s0, s1};
             dst[(int64_t)g * 64] = v;
             apply_lut8_spread(step, order, s0, s1);
         }
         const u64x2_t v = {s0, s1};
-        dst[(int64_t)(kInitSteps - 1) * 64] = v;
+        dst[(int64_t)(steps - 1) * 64] = v;
         return;
     }
-    for (int g = 0; g < kInitSteps; ++g) {
+    for (int g = 0; g < steps; ++g) {
         if (first + (int64_t)g * 64 >= n)
             break;
         const int64_t idx = first + (int64_t)g * 64 + lane;
@@ -494,7 +446,7 @@ __global__ __launch_bounds__(kTabBlock) void init_states_tables_kernel(uint64_t 
             u64x2_t v = {s0, s1};
             *reinterpret_cast<u64x2_t *>(states + 2 * idx) = v;
         }
-        if (g + 1 < kInitSteps)
+        if (g + 1 < steps)
             apply_lut8_spread(step, order, s0, s1);
     }
 }
@@ -1187,22 +1139,22 @@ int nbh_xoro_init_states(void *states, int64_t n, uint64_t seed, uint64_t subseq
         return rc;
     hipStream_t hs = nbh_hip_stream(stream);
     nbh_stream_report report(hs);
-    if (n >= kTablesFrom) {
-        // one workgroup of 16 wavefronts per 65536 states, lookup tables in LDS
-        const int64_t per_block = (int64_t)(kTabBlock / 64) * 64 * kInitSteps;
-        const int64_t grid = (n + per_block - 1) / per_block;
-        if (grid > 0x7fffffffLL)
-            return (int)hipErrorInvalidValue;
-        const u64x2_t *lut = reinterpret_cast<const u64x2_t *>(dtable + (size_t)kPowers * 128);
-        const u64x2_t *lanes = lut + kLutEntries;
-        hipLaunchKernelGGL(init_states_tables_kernel, dim3((unsigned)grid), dim3(kTabBlock), 0, hs,
-                           (uint64_t *)states, n, base.s0, base.s1, dtable, lut, lanes);
-        return nbh_launch_status();
-    }
-    const int64_t per_block = (int64_t)(kInitBlock / 64) * 64 * kInitSteps;
+    // Steps per wavefront: as few as leave every SIMD of the device four wavefronts, 64 from 2^24
+    // states on (one workgroup of 16 wavefronts per compute unit and 65536 states then).
+    // Measured per launch, 64 steps whatever the size (and, below 2^18 states, masked XORs over
+    // the 128 columns instead of tables) -> this choice: 2^12 states 201 -> 7.7 us, 2^16 208 ->
+    // 10.1, 2^18 40 -> 12.5, 2^20 42 -> 17.5, 2^22 47 -> 27, 2^23 49 -> 37, 2^24 the same.
+    const int64_t wavefronts_wanted = (int64_t)nbh_cu_count() * (kTabBlock / 64);
+    int64_t steps = (n + 64 * wavefronts_wanted - 1) / (64 * wavefronts_wanted);
+    steps = steps < 1 ? 1 : steps > kInitSteps ? kInitSteps : steps;
+    const int64_t per_block = (int64_t)(kTabBlock / 64) * 64 * steps;
     const int64_t grid = (n + per_block - 1) / per_block;
-    hipLaunchKernelGGL(init_states_kernel, dim3((unsigned)grid), dim3(kInitBlock), 0, hs, (uint64_t *)states, n,
-                       base.s0, base.s1, dtable);
+    if (grid > 0x7fffffffLL)
+        return (int)hipErrorInvalidValue;
+    const u64x2_t *lut = reinterpret_cast<const u64x2_t *>(dtable + (size_t)kPowers * 128);
+    const u64x2_t *lanes = lut + kLutEntries;
+    hipLaunchKernelGGL(init_states_tables_kernel, dim3((unsigned)grid), dim3(kTabBlock), 0, hs, (uint64_t *)states,
+                       n, base.s0, base.s1, dtable, lut, lanes, (int)steps);
     return nbh_launch_status();
 }
 

@@ -43,7 +43,8 @@ def test_create_stream():
 @pytest.mark.parametrize("n,seed,start", [(1, 0, 0), (10, 1, 0), (63, 1, 1), (64, 42, 0), (65, 42, 5),
                                           (4095, 7, 2), (4097, 2**64 - 1, 0), (16385, -3, 9),
                                           (70001, 42, 0), (262143, 3, 1), (262144, 5, 2),
-                                          (300000, 12345678901234567890, 17), (1048576 + 4097, 8, 3)])
+                                          (300000, 12345678901234567890, 17), (1048576 + 4097, 8, 3),
+                                          (3 * 2**20 + 100, 11, 4), (2**23 - 5, 6, 1)])
 def test_states_bit_exact_against_sequential_chain(n, seed, start):
     _say("states", n, seed, start)
     got = cuda.random.create_xoroshiro128p_states(n, seed=seed, subsequence_start=start).copy_to_host()
