@@ -50,7 +50,7 @@ MEASURED_TRAFFIC = {
     "reduce_f32_functor": 1073931926,
     "rng_uniform_f32": 4831416814,
     "rng_normal_f64": 2684025959,
-    "rng_init": 298491702,
+    "rng_init": 298423381,
 }
 
 
