@@ -9,7 +9,7 @@
 //                  rounded double logarithm rounds to; u == 0 gives -infinity.
 //   bm_cos_2pi(x)  cosine of a double in [0, 6.2832], i.e. of 2*pi*u, within one unit
 //                  in the last place of double.
-//   bm_sqrt_pos(a) square root for the range that occurs.
+//   bm_neg_sqrt_of_neg(w)  -sqrt(-w) for the range that occurs, w = 2 log(u).
 //
 // The general-purpose library routines spend most of their time on cases that
 // cannot occur here (subnormals, huge arguments, Payne-Hanek reduction): on
@@ -50,7 +50,8 @@ BM_FN double fma_const(double a, double b, double c)
 // into 128 runs of 2^16; run j has a centre c_j (1.0 for the run that contains 1.0)
 // and the table holds q_j = RN(1 / c_j) and t_j = -log(q_j) as a double-double, so that
 //     log(m) = t_j + log1p(r),  r = m * q_j - 1  (|r| <= 2^-8)
-// holds exactly.  t_hi keeps 42 fractional bits: e * ln2_hi + t_hi is then exact.
+// holds exactly.  t_hi keeps 42 fractional bits: e * ln2_hi + t_hi is then exact.  (The table
+// words are stored doubled, for the evaluation of 2 log(u) below.)
 // Nothing is carried in two parts beyond that: a compensated evaluation (r as a sum of
 // two doubles, error-free addition of the leading terms) is good to 0.513 units in the
 // last place at 20 double-precision operations; the 12 below lose up to 4.5 where u is
@@ -86,8 +87,8 @@ inline void build_log_table(LogTable &t)
         const long double full = -logl((long double)q);
         const double hi_part = (double)(std::floor((double)full * 0x1p42) * 0x1p-42);
         t.q[j] = q;
-        t.t_hi[j] = hi_part;
-        t.t_lo[j] = (double)(full - (long double)hi_part);
+        t.t_hi[j] = 2.0 * hi_part;  // the table serves 2 log(u), see log2x_positive_f32
+        t.t_lo[j] = 2.0 * (double)(full - (long double)hi_part);
     }
     const double c[6] = {-0x1.8fae9be8838d4p-37, 0x1.1ee9ebdb4b1c4p-29, -0x1.27e4f809c52adp-22,
                          0x1.a01a019cb159p-16,   -0x1.6c16c16c15177p-10, 0x1.555555555554cp-5};
@@ -102,7 +103,10 @@ inline void build_log_table(LogTable &t)
 // `Tab` in the functions below: a pointer to a LogTable - `const LogTable *`, or on the device
 // one that carries the LDS address space, so that the look-ups are LDS instructions with
 // 32-bit addresses.
-template <typename Tab> BM_FN double log_positive_f32(float u, Tab tab)
+// Returns 2 log(u): the generators want -2 log(u), the doubling is exact in every step (table
+// words, coefficients and ln 2 carry the factor), and the sign is a source modifier where the
+// value is used - one multiplication less than doubling the rounded logarithm.
+template <typename Tab> BM_FN double log2x_positive_f32(float u, Tab tab)
 {
     uint32_t bits;
 #ifdef __HIP_DEVICE_COMPILE__
@@ -123,30 +127,34 @@ template <typename Tab> BM_FN double log_positive_f32(float u, Tab tab)
     const double m = (double)mf, fe = (double)e;
     // r = RN(m * q_j - 1): one rounding, relative to r itself
     const double r = __builtin_fma(m, tab->q[j], -1.0);
-    // log1p(r) - r, |r| <= 2^-8: the r^7 / 7 term is below 2^-58
-    double p = fma_const(r, -1.0 / 6.0, 1.0 / 5.0);
-    p = fma_const(r, p, -1.0 / 4.0);
-    p = fma_const(r, p, 1.0 / 3.0);
-    p = __builtin_fma(r, p, -0.5);
-    const double ln2_hi = 0x1.62e42feep-1;             // 32 bits of ln 2
-    const double ln2_lo = 0x1.a39ef35793c76p-33;       // ln 2 - ln2_hi
+    // 2 (log1p(r) - r), |r| <= 2^-8: the r^7 / 7 term is below 2^-58
+    double p = fma_const(r, -2.0 / 6.0, 2.0 / 5.0);
+    p = fma_const(r, p, -2.0 / 4.0);
+    p = fma_const(r, p, 2.0 / 3.0);
+    p = __builtin_fma(r, p, -1.0);
+    const double ln2_hi = 2.0 * 0x1.62e42feep-1;       // 32 bits of ln 2, doubled
+    const double ln2_lo = 2.0 * 0x1.a39ef35793c76p-33; // ln 2 - ln2_hi, doubled
     const double hi = __builtin_fma(fe, ln2_hi, tab->t_hi[j]);  // exact
     const double lo = __builtin_fma(r * r, p, __builtin_fma(fe, ln2_lo, tab->t_lo[j]));
-    return hi + (r + lo);                              // the small terms first
+    return hi + __builtin_fma(r, 2.0, lo);             // the small terms first
 }
 
 template <typename Tab> BM_FN double bm_log_f32(float u, Tab tab)
 {
-    const double v = log_positive_f32(u, tab);
+    const double v = 0.5 * log2x_positive_f32(u, tab);
     return (u == 0.0f) ? -HUGE_VAL : v;
 }
 
-// What the generators use: the logarithm rounded to float32.  The case u == 0 is sorted out
-// after the rounding, on one 32-bit word instead of two.
+// What the generators use: 2 log(u) rounded to float32, which is twice the float32 the logarithm
+// rounds to.  The case u == 0 is sorted out after the rounding, on one 32-bit word instead of two.
+template <typename Tab> BM_FN float bm_log2x_f32_rounded(float u, Tab tab)
+{
+    const float v = (float)log2x_positive_f32(u, tab);
+    return (u == 0.0f) ? -HUGE_VALF : v;
+}
 template <typename Tab> BM_FN float bm_log_f32_rounded(float u, Tab tab)
 {
-    const float v = (float)log_positive_f32(u, tab);
-    return (u == 0.0f) ? -HUGE_VALF : v;
+    return 0.5f * bm_log2x_f32_rounded(u, tab);
 }
 
 // ---- cosine ------------------------------------------------------------------------
@@ -165,14 +173,24 @@ template <typename Tab> BM_FN float bm_log_f32_rounded(float u, Tab tab)
 // instructions are what bounds the generators, so ONE Horner chain runs: the quadrant
 // picks factor, tail and base per lane (32-bit selects) and the row of the coefficient
 // table (loads from LDS on the device, which cost the vector ALU nothing).
-template <typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
+// NEGATED: the cosine with its sign flipped, at no cost (the quadrant's sign bit is an added constant).
+template <bool NEGATED = false, typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
 {
     const double inv_pio2 = 0x1.45f306dc9c883p-1;
     const double pio2_1 = 0x1.921fb544p+0;             // first 33 bits of pi/2
     const double pio2_2 = 0x1.0b4611a6p-34;            // next 33 bits
     const double pio2_2t = 0x1.3198a2e037073p-69;      // pi/2 - pio2_1 - pio2_2
-    const double fn = __builtin_rint(x * inv_pio2);
-    const int n = (int)fn;
+    // x * 2/pi rounded to an integer in one fused operation: added to 1.5 * 2^52 the product loses
+    // its fraction (to nearest, ties to even), and the integer stands in the low word of the sum
+    const double shifted = __builtin_fma(x, inv_pio2, 0x1.8p52);
+    const double fn = shifted - 0x1.8p52;
+#ifdef __HIP_DEVICE_COMPILE__
+    const int n = __double2loint(shifted);
+#else
+    int64_t shifted_bits;
+    std::memcpy(&shifted_bits, &shifted, 8);
+    const int n = (int)(uint32_t)shifted_bits;
+#endif
     const double t = __builtin_fma(-fn, pio2_1, x);    // exact: fn * pio2_1 has 36 bits
     const double y0 = __builtin_fma(-fn, pio2_2, t);   // fn * pio2_2 is exact too: one rounding, of t - fn * pio2_2
     // what that rounding lost (t - y0 is exact and so is the fused operation), less the third piece
@@ -203,11 +221,11 @@ template <typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
 #ifdef __HIP_DEVICE_COMPILE__
     // bit 1 of n + 1 moved onto the sign bit and xor-ed in: a shift-and-add and one
     // three-input bit operation, hi ^ (sign & 0x80000000)
-    const uint32_t sign = ((uint32_t)n << 30) + 0x40000000u;
+    const uint32_t sign = ((uint32_t)n << 30) + (NEGATED ? 0xC0000000u : 0x40000000u);
     const uint32_t hi = (uint32_t)__builtin_amdgcn_bitop3_b32(__double2hiint(pick), sign, 0x80000000u, 0x78);
     return __hiloint2double((int)hi, __double2loint(pick));
 #else
-    return (((n + 1) & 2) != 0) ? -pick : pick;
+    return ((((n + 1) & 2) != 0) != NEGATED) ? -pick : pick;
 #endif
 }
 
@@ -221,22 +239,25 @@ template <typename Tab> BM_FN double bm_cos_2pi(double x, Tab tab)
 // the float64 normals over all 260 million values the first uniform can take.  Leaving h
 // as the estimate gave it would save an operation and leave an error near 2^-77: enough to
 // move the last bit of some thirty of those values.)
-// Zero and +infinity, where the estimate is infinite or zero, are told by one class test.
-BM_FN double bm_sqrt_pos(double a)
+// Zero and infinity, where the estimate is infinite or zero, are told by one class test.
+// The argument comes negated, w = 2 log(u) <= 0, and the root goes out negated: -sqrt(-w), and w
+// itself where that is a zero or -infinity.  Every negation below is an operand modifier of an
+// instruction that is there anyway; the caller multiplies by the negated cosine.
+BM_FN double bm_neg_sqrt_of_neg(double w)
 {
 #ifdef __HIP_DEVICE_COMPILE__
-    const double y = __builtin_amdgcn_rsq(a);
-    double g = a * y;
+    const double y = __builtin_amdgcn_rsq(-w);
+    double g = -w * y;
     double h = 0.5 * y;
     const double r = __builtin_fma(-h, g, 0.5);
     g = __builtin_fma(g, r, g);
     h = __builtin_fma(h, r, h);
-    const double d = __builtin_fma(-g, g, a);
-    g = __builtin_fma(d, h, g);
-    constexpr int kZeroOrPlusInfinity = 0x020 | 0x040 | 0x200;  // -0, +0, +infinity
-    return __builtin_amdgcn_class(a, kZeroOrPlusInfinity) ? a : g;
+    const double d = __builtin_fma(-g, g, -w);
+    const double neg_g = __builtin_fma(-d, h, -g);
+    constexpr int kZeroOrMinusInfinity = 0x020 | 0x040 | 0x004;  // -0, +0, -infinity
+    return __builtin_amdgcn_class(w, kZeroOrMinusInfinity) ? w : neg_g;
 #else
-    return std::sqrt(a);
+    return (w == 0.0) ? w : -std::sqrt(-w);
 #endif
 }
 

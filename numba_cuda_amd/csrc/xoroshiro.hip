@@ -500,8 +500,8 @@ struct NormalF32 {
         const float u1 = UniformF32::draw(s0, s1);
         const float u2 = UniformF32::draw(s0, s1);
         const float two_pi = 6.283185307179586f;
-        const float lg = bm::bm_log_f32_rounded(u1, tab);
-        const float r = sqrtf(-2.0f * lg);
+        const float lg2 = bm::bm_log2x_f32_rounded(u1, tab);  // 2 log(u1), exactly twice the float32 logarithm
+        const float r = sqrtf(-lg2);
         const float c = (float)bm::bm_cos_2pi((double)(two_pi * u2), tab);
         return r * c;
     }
@@ -516,10 +516,12 @@ struct NormalF64 {
         const float u1 = UniformF32::draw(s0, s1);
         const float u2 = UniformF32::draw(s0, s1);
         const double two_pi = 6.283185307179586;
-        const float lg = bm::bm_log_f32_rounded(u1, tab);
-        const double r = bm::bm_sqrt_pos(-2.0 * (double)lg);
-        const double c = bm::bm_cos_2pi(two_pi * (double)u2, tab);
-        return r * c;
+        const float lg2 = bm::bm_log2x_f32_rounded(u1, tab);  // 2 log(u1), exactly twice the float32 logarithm
+        // (-sqrt(-2 log u1)) * (-cos(2 pi u2)): both factors negated, which costs nothing, where
+        // negating 2 log(u1) for the square root would cost an instruction
+        const double neg_r = bm::bm_neg_sqrt_of_neg((double)lg2);
+        const double neg_c = bm::bm_cos_2pi<true>(two_pi * (double)u2, tab);
+        return neg_r * neg_c;
     }
 };
 
@@ -610,10 +612,18 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(uint64_t *__restrict__
                 }
             }
         } else if (live) {
-            // transcendental-heavy draws stay in a rolled loop: unrolling sixteen
+            // transcendental-heavy draws stay in a loop, two to a turn: unrolling sixteen
             // inlined log/cos bodies only thrashes the instruction cache
+            int j = 0;
 #pragma unroll 1
-            for (int j = 0; j < m; ++j)
+            for (; j + 1 < m; j += 2) {  // two values per 16-byte write where the value is 8 bytes
+                VT two[2];
+                two[0] = Gen::draw(s0, s1, tab);
+                two[1] = Gen::draw(s0, s1, tab);
+                park[lane][j] = two[0];
+                park[lane][j + 1] = two[1];
+            }
+            if (j < m)
                 park[lane][j] = Gen::draw(s0, s1, tab);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
