@@ -48,8 +48,8 @@ MEASURED_TRAFFIC = {
     "reduce_i64_sum": 2147532373,
     "reduce_f32_sum_reference_order": 1073951990,
     "reduce_f32_functor": 1073931926,
-    "rng_uniform_f32": 4831416814,
-    "rng_normal_f64": 2684025959,
+    "rng_uniform_f32": 4831199483,
+    "rng_normal_f64": 2683917445,
     "rng_init": 298423381,
 }
 
