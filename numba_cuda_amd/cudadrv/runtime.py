@@ -1,26 +1,26 @@
-"""The runtime's version, under the names of the reference's
-numba/cuda/cudadrv/runtime.py:13-33 (there: the CUDA toolkit's version; here: the HIP
-runtime's, asked of the library)."""
+"""Version of the HIP runtime the library is linked against, under the names user code
+knows from the reference (numba/cuda/cudadrv/runtime.py:13-33, where they report the CUDA
+toolkit).  The numbers come from the GPU library (`nbh_hip_versions`); no device is needed."""
 
-from .driver import driver
+from . import driver as _driver
 
-# ROCm releases this package's kernels are built and tested with
+# major versions of ROCm whose HIP runtime the kernels are built and tested with
 SUPPORTED_TOOLKIT_MAJOR_VERSIONS = (6, 7)
 
 
 class Runtime:
+    """`cuda.runtime`: what runs underneath."""
+
+    tested_majors = frozenset(SUPPORTED_TOOLKIT_MAJOR_VERSIONS)
+
     def get_version(self):
-        """(major, minor) of the HIP runtime."""
-        return driver.hip_versions()[1]
+        _, of_runtime = _driver.driver.hip_versions()
+        return of_runtime                      # (major, minor)
 
     def is_supported_version(self):
-        """Whether the HIP runtime is a version this package is tested with."""
-        return self.get_version()[0] in SUPPORTED_TOOLKIT_MAJOR_VERSIONS
+        major, _minor = self.get_version()
+        return major in self.tested_majors
 
 
 runtime = Runtime()
-
-
-def get_version():
-    """The runtime's version as (major, minor)."""
-    return runtime.get_version()
+get_version = runtime.get_version
