@@ -58,6 +58,9 @@ typedef nbh_u32x4 u32x4;
 
 // Shape of the workgroup tile per item size: WR x WC wavefronts, REP wavefront
 // tiles stacked along the rows per wavefront.  A wavefront tile is 8V x 8V items.
+// (2-byte items, int16 8192 x 32768, us: 256 x 64 as below 186; 512 x 64 with eight wavefronts
+// 190, with four and REP = 2 200; 128 x 64 with REP = 2 196; 256 x 128 206; 128 x 128 222;
+// 128 x 256 193.)
 template <int E> struct ShapeOf;
 template <> struct ShapeOf<1> { static constexpr int WR = 4, WC = 1, REP = 1; };   // 512 x 128
 template <> struct ShapeOf<2> { static constexpr int WR = 4, WC = 1, REP = 1; };   // 256 x 64
