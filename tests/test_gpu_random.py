@@ -51,6 +51,20 @@ def test_states_bit_exact_against_sequential_chain(n, seed, start):
     np.testing.assert_array_equal(got, cref.init_states(n, seed, start))
 
 
+def test_states_of_random_sizes_seeds_and_starts():
+    """Sizes on both sides of every choice the launch makes (one step per wavefront up to 2^18
+    states, more above; whole and ragged last runs), random seeds and subsequence starts."""
+    rng = np.random.default_rng(77)
+    sizes = [int(rng.integers(1, 5000)) for _ in range(4)] + [int(rng.integers(5000, 300000)) for _ in range(4)] + \
+            [int(rng.integers(300000, 3000000)) for _ in range(4)] + [262145, 524288, 524289, 4096 * 64 * 3]
+    for n in sizes:
+        seed = int(rng.integers(0, 2**63)) * 2 + int(rng.integers(0, 2))
+        start = int(rng.integers(0, 2**20))
+        _say("states, random", n, seed, start)
+        got = cuda.random.create_xoroshiro128p_states(n, seed=seed, subsequence_start=start).copy_to_host()
+        np.testing.assert_array_equal(got, cref.init_states(n, seed, start))
+
+
 def test_huge_subsequence_start_is_consistent():
     """2^40+3 and 2^64-1 jumps cannot be walked sequentially; the chain property
     states[i+1] == jump(states[i]) and the shift property still pin them."""
