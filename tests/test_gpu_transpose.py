@@ -209,6 +209,13 @@ def test_fullsize_float32_16384_square():
     assert _same_bytes(back, a)
 
 
+def test_fullsize_int16_16384_square_in_diagonal_order():
+    """Both pitches 32 KiB: the workgroups take the tiles in diagonal order."""
+    a = np.random.default_rng(3).integers(-32768, 32767, (16384, 16384), dtype=np.int16, endpoint=True)
+    got = cuda.to_device(a).T.copy_to_host()
+    assert _same_bytes(got, a.T)
+
+
 def test_fullsize_float64_ragged_12345_by_6789():
     a = np.random.default_rng(2).random((12345, 6789))
     got = cuda.to_device(a).T.copy_to_host()
